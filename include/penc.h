@@ -1,0 +1,119 @@
+/*
+ * penc.h -- C ABI of the MI355X (gfx950) permutohedral-lattice hash encoding.
+ *
+ * One shared library (libpenc_hip.so) replaces the native half of the reference: the pybind11
+ * class `EncodingWrapper` with its methods `forward`, `backward`,
+ * `double_backward_from_positions` (reference: src/PyBridge.cxx:36-42,
+ * include/permutohedral_encoding/Encoding.cuh:162-188) and the host launchers behind them
+ * (reference: src/Encoding.cu:55-334).
+ *
+ * Conventions
+ *  - Plain pointers and sizes only.  Unless a parameter says "host", every pointer is DEVICE
+ *    memory of the GPU that is current on the calling thread; it is borrowed for the duration of
+ *    the enqueued work.  The library never allocates or frees device memory and keeps no state.
+ *  - All arrays are fp32, densely packed, row-major:
+ *        positions            [N][D]
+ *        lattice_values       [L][C][2]      (8-byte aligned)
+ *        scale_factor         [L][D]         (from penc_scale_factors)
+ *        random_shift         [L][D]
+ *        anneal_window        [L]
+ *        sliced_values        [L+E][2][N]    E = ceil(D/2) if concat_points else 0
+ *        grad_sliced_values   [L+E][2][N]    (levels >= L are ignored)
+ *        lattice_values_grad  [L][C][2]      (the reference returns this logical shape as a
+ *                                             permuted view of [L][2][C], src/Encoding.cu:141,204)
+ *        positions_grad       [N][D]         (the reference returns this logical shape as a
+ *                                             transposed view of [D][N], src/Encoding.cu:152,205)
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is enqueued and
+ *    the call returns without synchronising, like the reference's launches on the current stream.
+ *  - D = pos_dim in 2..8, nr_feat must be 2 (reference: Encoding.cuh:139-156 supports 2..7 / 2).
+ *  - Every function returns PENC_OK or one of the error codes below; penc_status_string() names it.
+ */
+#ifndef PENC_H_
+#define PENC_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PENC_OK 0
+#define PENC_ERR_NULL_POINTER 1        /* a required pointer is NULL */
+#define PENC_ERR_BAD_SIZE 2            /* N, L or C is not positive, or a product overflows 2^31 elements */
+#define PENC_ERR_UNSUPPORTED_POS_DIM 3 /* pos_dim outside 2..8 (reference: Encoding.cuh:155) */
+#define PENC_ERR_UNSUPPORTED_NR_FEAT 4 /* nr_feat != 2 (reference: Encoding.cuh:142) */
+#define PENC_ERR_MISALIGNED 5          /* lattice_values / lattice_values_grad not 8-byte aligned */
+#define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
+
+const char* penc_status_string(int status);
+
+/* Number of extra output levels that carry the raw positions when concat_points is set.
+ * Replaces: src/Encoding.cu:71-74 and src/pytorch_modules/modules.py:95-103. */
+int penc_extra_levels(int pos_dim, int nr_feat, int concat_points);
+
+/* scale_factor_out[l][i] = fp32(1/sqrt((i+1)(i+2))) / sigmas[l], a true fp32 division.
+ * Both arrays are HOST memory.
+ * Replaces: EncodingFixedParams::compute_scale_factor_tensor, Encoding.cuh:55-69. */
+int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* scale_factor_out);
+
+/* Slice: sliced_values[l][f][n] = sum over the D+1 simplex vertices of
+ * lattice_values[l][slot][f] * barycentric * anneal_window[l]; extra levels copy
+ * positions * points_scaling (zero-padded).
+ * Replaces: Encoding<D,2>::forward, src/Encoding.cu:55-108 (kernel forward_gpu,
+ * kernels/permutohedral_encoding/EncodingGPU.cuh:68-256). */
+int penc_forward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                 const float* positions, const float* lattice_values, const float* scale_factor,
+                 const float* random_shift, const float* anneal_window, float* sliced_values,
+                 int concat_points, float points_scaling, void* stream);
+
+/* First backward.  lattice_values_grad and positions_grad are each optional (NULL = not wanted,
+ * the reference's require_*_grad flags); at least one must be given.  lattice_values_grad is
+ * cleared by the library before the scatter-add; positions_grad is written, not accumulated.
+ * Replaces: Encoding<D,2>::backward, src/Encoding.cu:112-215 (kernels backward_gpu and
+ * backward_gpu_only_pos, EncodingGPU.cuh:259-414 and 530-769). */
+int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                  const float* positions, const float* lattice_values, const float* scale_factor,
+                  const float* random_shift, const float* anneal_window,
+                  const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
+                  void* stream);
+
+/* Double backward from d(loss)/d(positions_grad): gradient w.r.t. lattice_values and w.r.t.
+ * grad_sliced_values ([L+E][2][N], zeros in the extra levels).  Either output may be NULL.
+ * lattice_values_grad is cleared by the library first.
+ * Replaces: Encoding<D,2>::double_backward_from_positions, src/Encoding.cu:219-334 (kernels
+ * double_backward_from_positions_gpu_1 / _2, EncodingGPU.cuh:1016-1257 and 1260-1493). */
+int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
+                                        int capacity, const float* positions,
+                                        const float* lattice_values, const float* scale_factor,
+                                        const float* random_shift, const float* anneal_window,
+                                        const float* double_positions_grad,
+                                        const float* grad_sliced_values, float* lattice_values_grad,
+                                        float* grad_grad_sliced_values, int concat_points, void* stream);
+
+/* Introspection for parity checks: what the kernels derive from each (level, point) before they
+ * touch the table.  Outputs are [L][N][D+1]; each may be NULL.
+ *   rem0, rank : the remainder-0 lattice point and the residual ranks after the hyperplane wrap
+ *   slot       : hashed table index of each of the D+1 vertices
+ *   barycentric: the D+1 interpolation weights
+ * Uses the same device code as the kernels above (reference: EncodingGPU.cuh:130-223). */
+int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
+                       const float* positions, const float* scale_factor, const float* random_shift,
+                       int* rem0, int* rank, int* slot, float* barycentric, void* stream);
+
+/* Memory-system probes used by the benchmark to measure the rooflines the encoding is priced
+ * against; they have no counterpart in the reference.
+ *   copy   : dst[i] = src[i] for n_float4 16-byte elements (streaming bandwidth, and the known-size
+ *            kernel that hardware byte counters are scaled by)
+ *   gather : every thread sums `per_thread` independent 8-byte loads table[idx[...]] and writes one
+ *            8-byte result; idx holds n_threads*per_thread precomputed slots
+ *   scatter: every thread issues `per_thread` pairs of fp32 atomic adds at table[idx[...]] */
+int penc_probe_copy(const float* src, float* dst, int64_t n_float4, void* stream);
+int penc_probe_gather(const float* table, const int* idx, int64_t n_threads, int per_thread,
+                      float* out, void* stream);
+int penc_probe_scatter(float* table, const int* idx, int64_t n_threads, int per_thread, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* PENC_H_ */

@@ -1,0 +1,250 @@
+"""ctypes binding over ``libpenc_hip.so`` (the C ABI declared in ``include/penc.h``).
+
+This is the only way the package computes anything: there is no CPU or pure-PyTorch fallback.
+If the library is missing or a tensor is not on a GPU the call raises.
+
+The classes ``EncodingInput``, ``EncodingFixedParams`` and ``EncodingWrapper`` mirror the three
+classes the reference exposes through pybind11 (``src/PyBridge.cxx:20-42``) so that the autograd
+functions and the module read like the reference's.
+"""
+import ctypes
+import os
+
+import numpy as np
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpenc_hip.so")
+_lib = None
+
+_c_f32p = ctypes.c_void_p
+_SIGNATURES = {
+    "penc_status_string": (ctypes.c_char_p, [ctypes.c_int]),
+    "penc_extra_levels": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "penc_scale_factors": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p]),
+    "penc_forward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                    _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                    ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
+    "penc_backward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                     _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                     ctypes.c_void_p]),
+    "penc_double_backward_from_positions": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                                           ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                                           _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int,
+                                                           ctypes.c_void_p]),
+    "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
+                                          _c_f32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, _c_f32p,
+                                          ctypes.c_void_p]),
+    "penc_probe_copy": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_void_p]),
+    "penc_probe_gather": (ctypes.c_int, [_c_f32p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, _c_f32p,
+                                         ctypes.c_void_p]),
+    "penc_probe_scatter": (ctypes.c_int, [_c_f32p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def lib():
+    """Loads the library once; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m permutohedral_encoding_amd.build` "
+                "(there is no fallback implementation)")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = handle
+    return _lib
+
+
+def _check(status, what):
+    if status != 0:
+        msg = lib().penc_status_string(status).decode()
+        raise RuntimeError(f"{what}: {msg} (status {status})")
+
+
+def extra_levels(pos_dim, nr_feat, concat_points):
+    return int(lib().penc_extra_levels(int(pos_dim), int(nr_feat), int(bool(concat_points))))
+
+
+def scale_factors(pos_dim, sigmas):
+    """Host computation of the (L, D) scale-factor table (reference: Encoding.cuh:55-69)."""
+    sig = np.ascontiguousarray(np.asarray(sigmas, dtype=np.float32).reshape(-1))
+    out = np.empty((sig.size, int(pos_dim)), np.float32)
+    _check(lib().penc_scale_factors(int(pos_dim), int(sig.size), sig.ctypes.data, out.ctypes.data), "scale_factors")
+    return out
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _require(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_f32_gpu(t, name, ndim):
+    _require(isinstance(t, torch.Tensor), f"{name} must be a torch.Tensor")
+    _require(t.is_cuda, f"{name} should be in GPU memory. Please call .cuda() on the tensor")
+    _require(t.dtype == torch.float32, f"{name} should be of type float")
+    _require(t.dim() == ndim, f"{name} should have {ndim} dimensions, however it has sizes {tuple(t.shape)}")
+
+
+class EncodingInput:
+    """Per-call inputs (reference: ``EncodingInput``, include/permutohedral_encoding/Encoding.cuh:14-29)."""
+
+    def __init__(self, lattice_values, positions_raw, anneal_window, require_lattice_values_grad, require_positions_grad):
+        self.m_lattice_values = lattice_values
+        self.m_positions_raw = positions_raw
+        self.m_anneal_window = anneal_window
+        self.m_require_lattice_values_grad = bool(require_lattice_values_grad)
+        self.m_require_positions_grad = bool(require_positions_grad)
+
+
+class EncodingFixedParams:
+    """Parameters fixed for the lifetime of an encoding (reference: ``EncodingFixedParams``, Encoding.cuh:31-70).
+
+    Holds the random-shift tensor by handle, so an in-place update of the parameter (``load_state_dict``)
+    is seen by later calls, and owns the scale-factor table.
+    """
+
+    def __init__(self, pos_dim, capacity, nr_levels, nr_feat_per_level, sigmas_list, random_shift_per_level,
+                 concat_points, points_scaling):
+        self.m_pos_dim = int(pos_dim)
+        self.m_capacity = int(capacity)
+        self.m_nr_levels = int(nr_levels)
+        self.m_nr_feat_per_level = int(nr_feat_per_level)
+        self.m_sigmas_list = [float(s) for s in np.asarray(sigmas_list, dtype=np.float32).reshape(-1)]
+        self.m_random_shift_per_level = random_shift_per_level
+        self.m_concat_points = bool(concat_points)
+        self.m_points_scaling = float(points_scaling)
+        sf = scale_factors(self.m_pos_dim, self.m_sigmas_list)
+        self.m_scale_factor = torch.from_numpy(sf).to(random_shift_per_level.device)
+
+
+class EncodingWrapper:
+    """The native encoding object (reference: ``EncodingWrapper``, Encoding.cuh:162-188)."""
+
+    def __init__(self, pos_dim, nr_feat_per_level, fixed_params):
+        if nr_feat_per_level != 2:
+            raise RuntimeError("Encoding: nr_feat_per_level must be 2 since other values are not yet implemented")
+        if pos_dim not in (2, 3, 4, 5, 6, 7, 8):
+            raise RuntimeError("Encoding: pos_dim must be 2,3,4,5,6,7 or 8")
+        self.pos_dim = int(pos_dim)
+        self.nr_feat = int(nr_feat_per_level)
+        self.fixed_params = fixed_params
+
+    @staticmethod
+    def create(pos_dim, nr_feat_per_level, fixed_params):
+        return EncodingWrapper(pos_dim, nr_feat_per_level, fixed_params)
+
+    # -- checks shared by the three calls (reference: src/Encoding.cu:38-45, 57-66, 119-125)
+    def _check_common(self, inp):
+        fp = self.fixed_params
+        pos, lv, win = inp.m_positions_raw, inp.m_lattice_values, inp.m_anneal_window
+        _check_f32_gpu(pos, "positions", 2)
+        _require(pos.shape[0] != 0, "Why do we have 0 points")
+        _require(pos.shape[1] == fp.m_pos_dim,
+                 f"Pos dim for the lattice doesn't correspond with the position of the points. Lattice was initialized "
+                 f"with {fp.m_pos_dim} and points have pos dim {pos.shape[1]}")
+        _check_f32_gpu(lv, "lattice_values", 3)
+        _require(lv.is_contiguous(), "lattice_values must be contiguous (two floats are loaded at a time)")
+        _require(lv.shape[2] == self.nr_feat, "lattice_values should be nr_levels x capacity x 2")
+        levels = lv.shape[0]
+        shift = fp.m_random_shift_per_level
+        _check_f32_gpu(shift, "random_shift_per_level", 2)
+        _require(shift.shape[0] == levels,
+                 "Random shift should have the first dimension the same as the nr of resolutions")
+        _require(shift.shape[1] == fp.m_pos_dim, "Random shift should have the second dimension the same as the pos dim")
+        _check_f32_gpu(win, "anneal_window", 1)
+        _require(win.shape[0] == levels, "anneal_window should have the first dimension the same as the nr of resolutions")
+        _require(fp.m_scale_factor.shape == (levels, fp.m_pos_dim), "scale list should have one entry per level")
+        dev = pos.device
+        for t, name in ((lv, "lattice_values"), (shift, "random_shift_per_level"), (win, "anneal_window")):
+            _require(t.device == dev, f"{name} must be on the same device as positions")
+        if fp.m_scale_factor.device != dev:
+            fp.m_scale_factor = fp.m_scale_factor.to(dev)
+        return pos.contiguous(), lv, shift.contiguous(), win.contiguous(), levels, lv.shape[1]
+
+    def _check_grad(self, grad, levels, extra, n):
+        _check_f32_gpu(grad, "grad_sliced_values_monolithic", 3)
+        _require(grad.is_contiguous(), "Grad sliced values needs to be contiguous. Please call .contiguous() on it")
+        _require(grad.shape == (levels + extra, self.nr_feat, n),
+                 "grad_sliced_values_monolithic should be nr_resolutions x val_dim x nr_positions")
+
+    def forward(self, inp):
+        """-> sliced values (L+E, 2, N)  (reference: Encoding<D,2>::forward, src/Encoding.cu:55-108)."""
+        fp = self.fixed_params
+        pos, lv, shift, win, levels, cap = self._check_common(inp)
+        n = pos.shape[0]
+        extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
+        out = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
+        with torch.cuda.device(pos.device):
+            _check(lib().penc_forward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                                      _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(out),
+                                      int(fp.m_concat_points), fp.m_points_scaling, _stream()), "forward")
+        return out
+
+    def backward(self, inp, grad_sliced_values_monolithic):
+        """-> (lattice_values_grad (L,C,2) or None, positions_grad (N,D) or None)
+        (reference: Encoding<D,2>::backward, src/Encoding.cu:112-215)."""
+        fp = self.fixed_params
+        pos, lv, shift, win, levels, cap = self._check_common(inp)
+        n = pos.shape[0]
+        extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
+        self._check_grad(grad_sliced_values_monolithic, levels, extra, n)
+        lv_grad = torch.empty_like(lv) if inp.m_require_lattice_values_grad else None
+        pos_grad = torch.empty_like(pos) if inp.m_require_positions_grad else None
+        if lv_grad is None and pos_grad is None:
+            return None, None
+        with torch.cuda.device(pos.device):
+            _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                                       _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
+                                       _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(pos_grad), _stream()),
+                   "backward")
+        return lv_grad, pos_grad
+
+    def double_backward_from_positions(self, inp, double_positions_grad, grad_sliced_values_monolithic):
+        """-> (lattice_values_grad (L,C,2), grad_grad_sliced_values (L+E,2,N))
+        (reference: Encoding<D,2>::double_backward_from_positions, src/Encoding.cu:219-334)."""
+        fp = self.fixed_params
+        pos, lv, shift, win, levels, cap = self._check_common(inp)
+        n = pos.shape[0]
+        extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
+        self._check_grad(grad_sliced_values_monolithic, levels, extra, n)
+        _check_f32_gpu(double_positions_grad, "double_positions_grad", 2)
+        _require(double_positions_grad.shape == pos.shape, "double_positions_grad should be nr_positions x pos_dim")
+        dpos = double_positions_grad.contiguous()
+        lv_grad = torch.empty_like(lv)
+        ggs = torch.empty_like(grad_sliced_values_monolithic)
+        with torch.cuda.device(pos.device):
+            _check(lib().penc_double_backward_from_positions(
+                self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                _ptr(win), _ptr(dpos), _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(ggs),
+                int(fp.m_concat_points), _stream()), "double_backward_from_positions")
+        return lv_grad, ggs
+
+    def simplex_debug(self, positions, capacity):
+        """Introspection: dict(rem0, rank, slot (int32), barycentric) each of shape (L, N, D+1)."""
+        fp = self.fixed_params
+        _check_f32_gpu(positions, "positions", 2)
+        pos = positions.contiguous()
+        n, levels = pos.shape[0], fp.m_scale_factor.shape[0]
+        shape = (levels, n, self.pos_dim + 1)
+        out = {k: torch.empty(shape, dtype=torch.int32, device=pos.device) for k in ("rem0", "rank", "slot")}
+        out["barycentric"] = torch.empty(shape, dtype=torch.float32, device=pos.device)
+        shift = fp.m_random_shift_per_level.contiguous()
+        with torch.cuda.device(pos.device):
+            _check(lib().penc_simplex_debug(self.pos_dim, n, levels, int(capacity), _ptr(pos),
+                                            _ptr(fp.m_scale_factor.to(pos.device)), _ptr(shift), _ptr(out["rem0"]),
+                                            _ptr(out["rank"]), _ptr(out["slot"]), _ptr(out["barycentric"]), _stream()),
+                   "simplex_debug")
+        return out

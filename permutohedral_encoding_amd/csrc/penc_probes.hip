@@ -1,0 +1,105 @@
+// Memory-system probes: the rooflines the encoding kernels are priced against are measured, on
+// the same GPU and in the same run, with kernels that do nothing but the memory operation in
+// question.  None of this has a counterpart in the reference.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/penc.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+__global__ void __launch_bounds__(kBlock) copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, size_t n4) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
+}
+
+// `per_thread` independent 8-byte loads per thread, indices coalesced across the wave
+// (idx[k][thread]), one 8-byte store: the access pattern of the forward pass without its arithmetic.
+template <int K>
+__global__ void __launch_bounds__(kBlock) gather_kernel(const float2* __restrict__ table, const int* __restrict__ idx,
+                                                       size_t n_threads, float2* __restrict__ out) {
+    const size_t t = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= n_threads) return;
+    int slot[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) slot[k] = idx[k * n_threads + t];
+    float2 v[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) v[k] = table[slot[k]];
+    float2 acc = make_float2(0.0f, 0.0f);
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        acc.x += v[k].x;
+        acc.y += v[k].y;
+    }
+    out[t] = acc;
+}
+
+template <int K>
+__global__ void __launch_bounds__(kBlock) scatter_kernel(float* __restrict__ table, const int* __restrict__ idx,
+                                                        size_t n_threads) {
+    const size_t t = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if (t >= n_threads) return;
+    int slot[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) slot[k] = idx[k * n_threads + t];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        float* p = table + 2 * static_cast<size_t>(slot[k]);
+        __hip_atomic_fetch_add(p, 1.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_fetch_add(p + 1, 1.0f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+inline int check_launch() { return hipGetLastError() == hipSuccess ? PENC_OK : PENC_ERR_LAUNCH; }
+
+}  // namespace
+
+extern "C" {
+
+int penc_probe_copy(const float* src, float* dst, int64_t n_float4, void* stream) {
+    if (!src || !dst) return PENC_ERR_NULL_POINTER;
+    if (n_float4 <= 0) return PENC_ERR_BAD_SIZE;
+    const int64_t want = (n_float4 + kBlock * 4 - 1) / (kBlock * 4);
+    const unsigned blocks = static_cast<unsigned>(want < 16384 ? want : 16384);
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<const float4*>(src), reinterpret_cast<float4*>(dst), static_cast<size_t>(n_float4));
+    return check_launch();
+}
+
+#define PENC_PROBE_K(K_, ...)                                   \
+    switch (K_) {                                               \
+        case 1: { constexpr int KK = 1; __VA_ARGS__; } break;   \
+        case 2: { constexpr int KK = 2; __VA_ARGS__; } break;   \
+        case 3: { constexpr int KK = 3; __VA_ARGS__; } break;   \
+        case 4: { constexpr int KK = 4; __VA_ARGS__; } break;   \
+        case 5: { constexpr int KK = 5; __VA_ARGS__; } break;   \
+        case 6: { constexpr int KK = 6; __VA_ARGS__; } break;   \
+        case 7: { constexpr int KK = 7; __VA_ARGS__; } break;   \
+        case 8: { constexpr int KK = 8; __VA_ARGS__; } break;   \
+        case 9: { constexpr int KK = 9; __VA_ARGS__; } break;   \
+        default: return PENC_ERR_BAD_SIZE;                      \
+    }
+
+int penc_probe_gather(const float* table, const int* idx, int64_t n_threads, int per_thread, float* out, void* stream) {
+    if (!table || !idx || !out) return PENC_ERR_NULL_POINTER;
+    if (n_threads <= 0) return PENC_ERR_BAD_SIZE;
+    const dim3 grid(static_cast<unsigned>((n_threads + kBlock - 1) / kBlock));
+    PENC_PROBE_K(per_thread, hipLaunchKernelGGL((gather_kernel<KK>), grid, dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                                                reinterpret_cast<const float2*>(table), idx, static_cast<size_t>(n_threads),
+                                                reinterpret_cast<float2*>(out)));
+    return check_launch();
+}
+
+int penc_probe_scatter(float* table, const int* idx, int64_t n_threads, int per_thread, void* stream) {
+    if (!table || !idx) return PENC_ERR_NULL_POINTER;
+    if (n_threads <= 0) return PENC_ERR_BAD_SIZE;
+    const dim3 grid(static_cast<unsigned>((n_threads + kBlock - 1) / kBlock));
+    PENC_PROBE_K(per_thread, hipLaunchKernelGGL((scatter_kernel<KK>), grid, dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                                                table, idx, static_cast<size_t>(n_threads)));
+    return check_launch();
+}
+
+}  // extern "C"

@@ -30,3 +30,25 @@ def assert_sum_close(got, want64, abs64, rel=1e-4, what=""):
     bound = rel * abs64 + 1e-30
     worst = np.max(err / bound)
     assert worst <= 1.0, f"{what}: max err/bound = {worst:.3g} (rel {rel} of sum|terms|)"
+
+
+# ----------------------------------------------------------------------------- GPU side
+
+def make_encoding(pos_dim, sigmas, shift, concat_points=False, points_scaling=1.0, device="cuda"):
+    """The native encoding handle (C ABI via ctypes) for a given geometry, plus its fixed parameters."""
+    import torch
+    from permutohedral_encoding_amd import _native
+    shift_t = torch.from_numpy(np.ascontiguousarray(shift, dtype=np.float32)).to(device)
+    fp = _native.EncodingFixedParams(pos_dim, 0, len(sigmas), 2, sigmas, shift_t, concat_points, points_scaling)
+    return _native.EncodingWrapper.create(pos_dim, 2, fp), fp
+
+
+def to_gpu(a, device="cuda"):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device)
+
+
+def gpu_input(p, need_table_grad=True, need_pos_grad=True, device="cuda"):
+    from permutohedral_encoding_amd import _native
+    return _native.EncodingInput(to_gpu(p["table"], device), to_gpu(p["pos"], device), to_gpu(p["window"], device),
+                                 need_table_grad, need_pos_grad)

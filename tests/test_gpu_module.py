@@ -1,0 +1,112 @@
+"""The PyTorch surface on the GPU: module forward layout, autograd backward and double backward
+(eikonal-style), checked against the oracle through the chain rule."""
+import numpy as np
+import pytest
+
+from helpers import to_gpu
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+orc = pytest.importorskip("oracle.api")
+
+
+def make_module(d=3, cap=1 << 12, levels=6, **kw):
+    import permutohedral_encoding_amd as pe
+    torch.manual_seed(0)
+    m = pe.PermutoEncoding(d, cap, levels, 2, np.geomspace(1.0, 1e-2, levels), **kw)
+    with torch.no_grad():
+        m.lattice_values.uniform_(-1, 1)
+    return m
+
+
+def oracle_args(m, pos):
+    sf = orc.scale_factors(m.pos_dim, m.scale_per_level)
+    return (pos.detach().cpu().numpy(), m.lattice_values.detach().cpu().numpy(), sf,
+            m.random_shift_per_level.detach().cpu().numpy())
+
+
+def test_forward_layout_and_no_grad():
+    m = make_module()
+    pos = torch.rand(1000, 3, device="cuda")
+    with torch.no_grad():
+        out = m(pos)
+    assert out.shape == (1000, m.output_dims()) and out.is_contiguous()
+    p, t, sf, sh = oracle_args(m, pos)
+    want = orc.forward(p, t, sf, sh, np.ones(6, np.float32))  # (L,2,N)
+    want = want.transpose(2, 0, 1).reshape(1000, -1)  # column = level*2 + feat
+    assert np.allclose(out.cpu().numpy(), want, rtol=1e-5, atol=1e-6)
+    with pytest.raises(RuntimeError):
+        out.sum().backward()
+
+
+def test_backward_through_autograd():
+    m = make_module()
+    pos = torch.rand(2000, 3, device="cuda", requires_grad=True)
+    win = torch.tensor([1, 1, 1, 0.5, 0, 0], dtype=torch.float32)
+    out = m(pos, win)
+    up = torch.randn_like(out)
+    (out * up).sum().backward()
+    p, t, sf, sh = oracle_args(m, pos)
+    g = up.cpu().numpy().reshape(2000, 6, 2).transpose(1, 2, 0)
+    w = win.numpy()
+    wt = orc.backward_table(p, sf, sh, w, g, m.capacity, want_abs=True)
+    assert m.lattice_values.grad.shape == m.lattice_values.shape
+    err = np.abs(m.lattice_values.grad.cpu().numpy() - wt["grad64"])
+    assert np.all(err <= 1e-4 * wt["abs64"] + 1e-30)
+    wp = orc.backward_pos(p, t, sf, sh, w, g)["grad64"]
+    assert np.allclose(pos.grad.cpu().numpy(), wp, rtol=1e-4, atol=1e-4 * np.abs(wp).max())
+
+
+def test_double_backward_eikonal_style():
+    """loss = sum_n (|d(sum_c out[n,c]*a[c]) / d pos_n| - 1)^2 ; its gradient w.r.t. the table goes
+    through the double-backward kernels."""
+    m = make_module(levels=4)
+    n = 1500
+    pos = torch.rand(n, 3, device="cuda", requires_grad=True)
+    a = torch.randn(m.output_dims(), device="cuda")
+    out = m(pos)
+    sdf = (out * a).sum(dim=1)
+    grad_pos, = torch.autograd.grad(sdf.sum(), pos, create_graph=True)
+    loss = ((grad_pos.norm(dim=1) - 1.0) ** 2).sum()
+    loss.backward()
+    # chain rule by hand with the oracle: q = dloss/dgrad_pos, then table gradient of <q, posgrad(T, g)>
+    p, t, sf, sh = oracle_args(m, pos)
+    g = np.broadcast_to(a.cpu().numpy()[None], (n, m.output_dims())).reshape(n, 4, 2).transpose(1, 2, 0).copy()
+    w = np.ones(4, np.float32)
+    gp = orc.backward_pos(p, t, sf, sh, w, g)["grad64"]
+    assert np.allclose(grad_pos.detach().cpu().numpy(), gp, rtol=1e-4, atol=1e-4 * np.abs(gp).max())
+    nrm = np.linalg.norm(gp, axis=1, keepdims=True)
+    q = (2.0 * (nrm - 1.0) * gp / nrm).astype(np.float32)
+    r = orc.double_backward(p, t, sf, sh, w, q, g, want_abs=True)
+    err = np.abs(m.lattice_values.grad.cpu().numpy() - r["grad64"])
+    assert np.all(err <= 1e-3 * r["abs64"] + 1e-6 * np.abs(r["grad64"]).max())
+    # positions get no second-order gradient: the interpolant is piecewise linear
+    assert pos.grad is None or torch.all(pos.grad == 0)
+
+
+def test_state_dict_round_trip_and_pickle():
+    import pickle
+    m = make_module()
+    sd = m.state_dict()
+    assert set(sd) == {"lattice_values", "random_shift_per_level"}
+    m2 = make_module()
+    with torch.no_grad():
+        m2.random_shift_per_level.add_(1.0)
+    m2.load_state_dict(sd)
+    pos = torch.rand(500, 3, device="cuda")
+    with torch.no_grad():
+        assert torch.equal(m(pos), m2(pos))  # the native side sees the in-place update of the shift
+        m3 = pickle.loads(pickle.dumps(m))
+        assert torch.equal(m(pos), m3(pos))
+
+
+def test_concat_points_module():
+    m = make_module(concat_points=True, concat_points_scaling=0.1)
+    pos = torch.rand(300, 3, device="cuda", requires_grad=True)
+    out = m(pos)
+    assert out.shape == (300, 2 * (6 + 2)) == (300, m.output_dims())
+    assert torch.allclose(out[:, 12:15], pos.detach() * 0.1)
+    assert torch.all(out[:, 15] == 0)
+    out.sum().backward()  # gradient does not flow to positions through the copied columns (as in the reference)
+    assert m.lattice_values.grad is not None

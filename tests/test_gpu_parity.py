@@ -1,0 +1,273 @@
+"""Parity of the HIP kernels (called through the C ABI) with the CPU oracle, on the same seeded inputs.
+
+Bars (stated by the task): simplex rank, remainder-0 point and hashed slots bit-exact; forward
+features within 1e-5 relative / 1e-6 absolute; atomically accumulated gradients within 1e-4
+relative (of the sum of the magnitudes of the accumulated terms, see helpers.assert_sum_close).
+"""
+import numpy as np
+import pytest
+
+from helpers import random_problem, assert_sum_close, make_encoding, gpu_input, to_gpu
+from permutohedral_encoding_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+orc = pytest.importorskip("oracle.api")
+
+DIMS = [2, 3, 4, 5, 6, 7, 8]
+FWD_RTOL, FWD_ATOL = 1e-5, 1e-6
+SUM_RTOL = 1e-4
+
+
+def workload_problem(name, n):
+    w = wl.WORKLOADS[name]
+    p = wl.make_inputs(w, nr_points=n)
+    p["sf"] = orc.scale_factors(w.pos_dim, p["sigmas"])
+    return w, p
+
+
+def check_forward(got, want):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    bound = FWD_ATOL + FWD_RTOL * np.abs(want.astype(np.float64))
+    assert np.all(err <= bound), f"forward: max err {err.max():.3g}, worst err/bound {np.max(err / bound):.3g}"
+
+
+# ----------------------------------------------------------------------------- simplex, slots
+
+@pytest.mark.parametrize("d", DIMS)
+def test_simplex_rank_and_slots_bit_exact_all_dims(d):
+    cap = (1 << 19) if d != 5 else 100003  # one non-power-of-two capacity
+    p = random_problem(d, 5000, 12, 4, seed=20 + d, sigma_range=(1.0, 1e-4))
+    sf = orc.scale_factors(d, p["sigmas"])
+    want = orc.simplex(p["pos"], sf, p["shift"], cap)
+    enc, fp = make_encoding(d, p["sigmas"], p["shift"])
+    assert np.array_equal(fp.m_scale_factor.cpu().numpy(), sf)
+    got = enc.simplex_debug(to_gpu(p["pos"]), cap)
+    for k in ("rem0", "rank", "slot"):
+        assert np.array_equal(got[k].cpu().numpy(), want[k]), k
+    # the weights are computed with the same operations in the same order
+    assert np.array_equal(got["barycentric"].cpu().numpy(), want["bary"])
+
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_simplex_bit_exact_on_benchmark_configs(name):
+    w, p = workload_problem(name, 1 << 14)
+    want = orc.simplex(p["pos"], p["sf"], p["shift"], w.capacity)
+    enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
+    got = enc.simplex_debug(to_gpu(p["pos"]), w.capacity)
+    for k in ("rem0", "rank", "slot"):
+        assert np.array_equal(got[k].cpu().numpy(), want[k]), k
+
+
+# ----------------------------------------------------------------------------- the five configs, reduced N
+
+@pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
+def test_config_all_phases_match_oracle(name):
+    w, p = workload_problem(name, 1 << 14)
+    enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    grad_t, dpos_t = to_gpu(p["grad"]), to_gpu(p["dpos"])
+
+    out = enc.forward(inp).cpu().numpy()
+    check_forward(out, orc.forward(p["pos"], p["table"], p["sf"], p["shift"], p["window"]))
+    if w.masked_top_levels:
+        assert np.all(out[w.nr_levels - w.masked_top_levels:] == 0.0)
+
+    tg, pg = enc.backward(inp, grad_t)
+    want = orc.backward_table(p["pos"], p["sf"], p["shift"], p["window"], p["grad"], w.capacity, want32=False, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+    del want
+    wantp = orc.backward_pos(p["pos"], p["table"], p["sf"], p["shift"], p["window"], p["grad"])["grad64"]
+    scale = np.abs(wantp).max(axis=1, keepdims=True)
+    assert np.all(np.abs(pg.cpu().numpy() - wantp) <= SUM_RTOL * (np.abs(wantp) + scale) + 1e-30)
+
+    tg2, ggs = enc.double_backward_from_positions(inp, dpos_t, grad_t)
+    want = orc.double_backward(p["pos"], p["table"], p["sf"], p["shift"], p["window"], p["dpos"], p["grad"],
+                               want32=False, want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient")
+    ggs = ggs.cpu().numpy()
+    lvl_scale = np.abs(want["ggs"]).max(axis=(1, 2), keepdims=True)
+    assert np.all(np.abs(ggs - want["ggs"]) <= SUM_RTOL * (np.abs(want["ggs"]) + lvl_scale) + 1e-30)
+
+
+@pytest.mark.parametrize("d", DIMS)
+def test_all_dims_all_phases_match_oracle(d):
+    cap = 1 << 12  # small table: heavy slot sharing
+    p = random_problem(d, 3000, 8, cap, seed=40 + d, sigma_range=(1.0, 1e-3))
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    check_forward(enc.forward(inp).cpu().numpy(), orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"]))
+    tg, pg = enc.backward(inp, to_gpu(p["grad"]))
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+    wantp = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])["grad64"]
+    scale = np.abs(wantp).max(axis=1, keepdims=True)
+    assert np.all(np.abs(pg.cpu().numpy() - wantp) <= SUM_RTOL * (np.abs(wantp) + scale))
+    tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient")
+    lvl_scale = np.abs(want["ggs"]).max(axis=(1, 2), keepdims=True)
+    assert np.all(np.abs(ggs.cpu().numpy() - want["ggs"]) <= SUM_RTOL * (np.abs(want["ggs"]) + lvl_scale))
+
+
+# ----------------------------------------------------------------------------- edge cases
+
+@pytest.mark.parametrize("n", [1, 63, 64, 65, 255, 256, 257, 4095, 4097, 10001])
+def test_ragged_point_counts(n):
+    d, cap = 3, 1 << 10
+    p = random_problem(d, n, 5, cap, seed=n, sigma_range=(1.0, 1e-2))
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    check_forward(enc.forward(inp).cpu().numpy(), orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"]))
+    tg, pg = enc.backward(inp, to_gpu(p["grad"]))
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+    tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient")
+    assert ggs.shape == (5, 2, n)
+
+
+@pytest.mark.parametrize("cap", [1, 2, 7, 1000, 100003])
+def test_unusual_capacities_and_total_collision(cap):
+    d = 4
+    p = random_problem(d, 2000, 6, cap, seed=cap, sigma_range=(1.0, 1e-3))
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    check_forward(enc.forward(inp).cpu().numpy(), orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"]))
+    tg, _ = enc.backward(inp, to_gpu(p["grad"]))
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+
+
+def test_concat_points_extra_levels():
+    for d in (2, 3, 4, 5):
+        p = random_problem(d, 777, 3, 256, seed=d)
+        sf = orc.scale_factors(d, p["sigmas"])
+        enc, _ = make_encoding(d, p["sigmas"], p["shift"], concat_points=True, points_scaling=0.5)
+        inp = gpu_input(p)
+        out = enc.forward(inp).cpu().numpy()
+        want = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"], concat_points=True, points_scaling=0.5)
+        assert out.shape == want.shape
+        check_forward(out, want)
+        assert np.array_equal(out[3:], want[3:])
+        extra = want.shape[0] - 3
+        grad = np.concatenate([p["grad"], np.ones((extra, 2, 777), np.float32)])
+        tg, pg = enc.backward(inp, to_gpu(grad))
+        w = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], 256, want_abs=True)
+        assert_sum_close(tg.cpu().numpy(), w["grad64"], w["abs64"], SUM_RTOL, "table gradient")
+        tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(grad))
+        assert ggs.shape == grad.shape and torch.all(ggs[3:] == 0)
+
+
+def test_masked_levels_are_exact_zeros_and_noops():
+    d, cap = 3, 1 << 12
+    p = random_problem(d, 5000, 6, cap, seed=77)
+    p["window"] = np.array([1, 1, 0.5, 0, 0, 0], np.float32)
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    out = enc.forward(inp)
+    assert torch.all(out[3:] == 0)
+    tg, pg = enc.backward(inp, to_gpu(p["grad"]))
+    assert torch.all(tg[3:] == 0) and not torch.all(tg[:3] == 0)
+    tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    assert torch.all(tg2[3:] == 0) and torch.all(ggs[3:] == 0)
+    wantp = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])["grad64"]
+    assert np.allclose(pg.cpu().numpy(), wantp, rtol=1e-4, atol=1e-4 * np.abs(wantp).max())
+
+
+def test_only_one_gradient_requested():
+    d, cap = 3, 1 << 10
+    p = random_problem(d, 1000, 4, cap, seed=5)
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    both = enc.backward(gpu_input(p), to_gpu(p["grad"]))
+    tg, none = enc.backward(gpu_input(p, True, False), to_gpu(p["grad"]))
+    assert none is None and torch.allclose(tg, both[0], rtol=1e-4, atol=1e-6)
+    none, pg = enc.backward(gpu_input(p, False, True), to_gpu(p["grad"]))
+    assert none is None and torch.equal(pg, both[1])
+    assert enc.backward(gpu_input(p, False, False), to_gpu(p["grad"])) == (None, None)
+
+
+def test_error_paths():
+    d, cap = 3, 64
+    p = random_problem(d, 10, 2, cap, seed=1)
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    from permutohedral_encoding_amd import _native
+    good = gpu_input(p)
+    with pytest.raises(ValueError, match="0 points"):
+        enc.forward(_native.EncodingInput(good.m_lattice_values, good.m_positions_raw[:0], good.m_anneal_window, True, True))
+    with pytest.raises(ValueError, match="Pos dim"):
+        enc.forward(_native.EncodingInput(good.m_lattice_values, to_gpu(np.zeros((4, 2), np.float32)), good.m_anneal_window, True, True))
+    with pytest.raises(ValueError, match="GPU memory"):
+        enc.forward(_native.EncodingInput(good.m_lattice_values, good.m_positions_raw.cpu(), good.m_anneal_window, True, True))
+    with pytest.raises(ValueError, match="type float"):
+        enc.forward(_native.EncodingInput(good.m_lattice_values, good.m_positions_raw.double(), good.m_anneal_window, True, True))
+    with pytest.raises(ValueError, match="anneal_window"):
+        enc.forward(_native.EncodingInput(good.m_lattice_values, good.m_positions_raw, good.m_anneal_window[:1], True, True))
+    with pytest.raises(ValueError, match="contiguous"):
+        enc.backward(good, to_gpu(p["grad"]).transpose(0, 1).contiguous().transpose(0, 1))
+    with pytest.raises(ValueError, match="contiguous"):
+        enc.forward(_native.EncodingInput(good.m_lattice_values.transpose(0, 1), good.m_positions_raw, good.m_anneal_window, True, True))
+    with pytest.raises(RuntimeError, match="pos_dim"):
+        _native.EncodingWrapper.create(9, 2, None)
+    with pytest.raises(RuntimeError, match="nr_feat_per_level"):
+        _native.EncodingWrapper.create(3, 4, None)
+    # strided positions are accepted (the reference indexes through accessors)
+    pos2 = to_gpu(np.concatenate([p["pos"], p["pos"]], axis=1))[:, :3]
+    out = enc.forward(_native.EncodingInput(good.m_lattice_values, pos2, good.m_anneal_window, True, True))
+    assert torch.equal(out, enc.forward(good))
+
+
+# ----------------------------------------------------------------------------- size-independent properties at full size
+
+@pytest.mark.parametrize("name", ["c2", "c3", "c4", "c5"])
+def test_full_size_adjoint_identities(name):
+    """forward is linear in the table and the position gradient bilinear in (table, grad): at the
+    full benchmark sizes, where the CPU oracle would take minutes,
+        <forward(T), g> = <T, table_grad(g)>
+        <q, pos_grad(T, g)> = <ggs(q, T), g> = <table_grad2(q, g), T>
+    must hold (fp64 dot products of the fp32 results)."""
+    w = wl.WORKLOADS[name]
+    p = wl.make_inputs(w)
+    enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    grad_t, dpos_t = to_gpu(p["grad"]), to_gpu(p["dpos"])
+    table = inp.m_lattice_values.double()
+
+    out = enc.forward(inp)
+    tg, pg = enc.backward(inp, grad_t)
+    lhs = torch.sum(out.double() * grad_t.double()).item()
+    rhs = torch.sum(tg.double() * table).item()
+    scale = torch.sum(torch.abs(out.double() * grad_t.double())).item()
+    assert abs(lhs - rhs) <= 1e-5 * scale, (lhs, rhs, scale)
+
+    tg2, ggs = enc.double_backward_from_positions(inp, dpos_t, grad_t)
+    a = torch.sum(dpos_t.double() * pg.double()).item()
+    b = torch.sum(ggs.double() * grad_t.double()).item()
+    c = torch.sum(tg2.double() * table).item()
+    scale2 = torch.sum(torch.abs(ggs.double() * grad_t.double())).item()
+    assert abs(a - b) <= 1e-4 * scale2 and abs(a - c) <= 1e-4 * scale2, (a, b, c, scale2)
+
+    # atomics make the summation order vary between runs; the result must not vary beyond rounding
+    tg_again, _ = enc.backward(inp, grad_t)
+    assert torch.allclose(tg, tg_again, rtol=1e-3, atol=1e-6 * tg.abs().max().item())
+    assert torch.equal(out, enc.forward(inp))
+
+
+def test_full_size_constant_table_gives_window():
+    w = wl.WORKLOADS["c2"]
+    p = wl.make_inputs(w, need=("shift", "pos"))
+    enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
+    from permutohedral_encoding_amd import _native
+    table = torch.empty((w.nr_levels, w.capacity, 2), device="cuda")
+    table[..., 0] = 2.0
+    table[..., 1] = -3.0
+    win = torch.linspace(0.1, 1.0, w.nr_levels, device="cuda")
+    out = enc.forward(_native.EncodingInput(table, to_gpu(p["pos"]), win, False, False))
+    assert torch.allclose(out[:, 0], (2.0 * win)[:, None].expand(-1, w.nr_points), rtol=1e-5)
+    assert torch.allclose(out[:, 1], (-3.0 * win)[:, None].expand(-1, w.nr_points), rtol=1e-5)

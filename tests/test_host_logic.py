@@ -1,0 +1,149 @@
+"""CPU-side checks: the C-ABI library loads and exports what include/penc.h declares, the host
+functions match their closed forms / the oracle, and the Python surface mirrors the reference's."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import permutohedral_encoding_amd as pe
+from permutohedral_encoding_amd import _native, workloads
+from oracle import api as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "penc.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return re.findall(r"\b(penc_\w+)\s*\(", text)
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert len(names) >= 9
+    handle = ctypes.CDLL(_native.LIB_PATH)
+    for n in names:
+        assert hasattr(handle, n), f"{n} is declared in include/penc.h but not exported"
+    assert set(names) == set(_native.EXPORTED_SYMBOLS)
+
+
+def test_status_strings_and_extra_levels():
+    lib = _native.lib()
+    assert lib.penc_status_string(0) == b"ok"
+    assert b"pos_dim" in lib.penc_status_string(3)
+    assert b"nr_feat_per_level must be 2" in lib.penc_status_string(4)
+    for d in range(2, 9):
+        assert _native.extra_levels(d, 2, False) == 0
+        assert _native.extra_levels(d, 2, True) == math.ceil(d / 2) == orc.extra_levels(d, True)
+
+
+def test_argument_validation_without_a_gpu():
+    """The entry points validate before they launch, so the error codes can be checked on a CPU-only host."""
+    lib = _native.lib()
+    z = ctypes.c_void_p(0)
+    buf = np.zeros(64, np.float32)
+    p = buf.ctypes.data
+    assert lib.penc_forward(9, 2, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 3
+    assert lib.penc_forward(1, 2, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 3
+    assert lib.penc_forward(3, 4, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 4
+    assert lib.penc_forward(3, 2, 0, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 2
+    assert lib.penc_forward(3, 2, 10, 0, 16, p, p, p, p, p, p, 0, 1.0, None) == 2
+    assert lib.penc_forward(3, 2, 10, 2, 0, p, p, p, p, p, p, 0, 1.0, None) == 2
+    assert lib.penc_forward(3, 2, 1 << 30, 24, 16, p, p, p, p, p, p, 0, 1.0, None) == 2
+    assert lib.penc_forward(3, 2, 10, 2, 16, z, p, p, p, p, p, 0, 1.0, None) == 1
+    assert lib.penc_forward(3, 2, 10, 2, 16, p, p + 4, p, p, p, p, 0, 1.0, None) == 5
+    assert lib.penc_backward(3, 2, 10, 2, 16, p, p, p, p, p, p, z, z, None) == 1
+    assert lib.penc_backward(3, 2, 10, 2, 16, p, z, p, p, p, p, z, p, None) == 1
+    assert lib.penc_double_backward_from_positions(3, 2, 10, 2, 16, p, p, p, p, p, p, p, z, z, 0, None) == 1
+    assert lib.penc_simplex_debug(3, 0, 2, 16, p, p, p, z, z, z, z, None) == 2
+    assert lib.penc_scale_factors(3, 2, z, p) == 1
+
+
+@pytest.mark.parametrize("d", range(2, 9))
+def test_scale_factors_match_oracle_and_closed_form(d):
+    sig = np.geomspace(1.0, 1e-4, 24).astype(np.float32)
+    sf = _native.scale_factors(d, sig)
+    assert np.array_equal(sf, orc.scale_factors(d, sig))
+    i = np.arange(d, dtype=np.float64)
+    want = 1.0 / (np.sqrt((i + 1) * (i + 2))[None, :] * sig.astype(np.float64)[:, None])
+    assert np.all(np.abs(sf - want) <= 1.5 * np.spacing(want.astype(np.float32)))
+
+
+def test_cosine_window_and_coarse2fine():
+    c2f = pe.Coarse2Fine(24)
+    win = c2f(16 / 24)
+    assert win.dtype == torch.float32 and win.shape == (24,)
+    assert torch.equal(win, torch.tensor([1.0] * 16 + [0.0] * 8))  # exactly, not approximately
+    assert c2f.get_last_t() == 16 / 24
+    assert torch.equal(c2f(1.0), torch.ones(24))
+    assert torch.equal(c2f(0.0), torch.zeros(24))
+    w = c2f(0.3)  # alpha = 7.2: levels 0..6 on, level 7 at 0.5*(1+cos(pi*0.2+pi)), rest off
+    assert torch.all(w[:7] == 1) and torch.all(w[8:] == 0)
+    assert abs(w[7].item() - 0.5 * (1 + math.cos(math.pi * 0.2 + math.pi))) < 1e-6
+    with pytest.raises(AssertionError):
+        c2f(1.5)
+    assert torch.equal(win, torch.from_numpy(workloads.anneal_window(workloads.WORKLOADS["c5"])))
+
+
+def test_map_range_val():
+    assert pe.map_range_val(5, 0, 10, 0.0, 1.0) == 0.5
+    assert pe.map_range_val(-3, 0, 10, 2.0, 4.0) == 2.0
+    assert pe.map_range_val(30, 0, 10, 2.0, 4.0) == 4.0
+    assert pe.map_range_val(2.5, 0, 10, 1.0, -1.0) == 0.5
+
+
+def test_module_surface_on_cpu():
+    torch.manual_seed(0)
+    m = pe.PermutoEncoding(3, 1 << 10, 6, 2, np.geomspace(1.0, 1e-2, 6), device="cpu")
+    sd = m.state_dict()
+    assert list(sd) == ["lattice_values", "random_shift_per_level"]
+    assert sd["lattice_values"].shape == (6, 1 << 10, 2) and sd["lattice_values"].is_contiguous()
+    assert sd["random_shift_per_level"].shape == (6, 3)
+    assert torch.equal(m.anneal_window, torch.ones(6))
+    assert m.output_dims() == 12
+    assert 0.5e-5 < m.lattice_values.std().item() < 2e-5 and abs(m.lattice_values.mean().item()) < 1e-6
+    assert 5 < m.random_shift_per_level.std().item() < 15
+    assert np.array_equal(m.fixed_params.m_scale_factor.numpy(), orc.scale_factors(3, np.geomspace(1.0, 1e-2, 6)))
+    m2 = pe.PermutoEncoding(5, 64, 2, 2, [1.0, 0.5], concat_points=True, device="cpu")
+    assert m2.output_dims() == 2 * (2 + 3)
+    # same RNG stream as the reference: values are drawn as (capacity, levels, feat) and permuted
+    torch.manual_seed(0)
+    want = (torch.randn(1 << 10, 6, 2) * 1e-5).permute(1, 0, 2).contiguous()
+    assert torch.equal(sd["lattice_values"], want)
+    # no CPU path: the forward refuses loudly instead of falling back
+    with pytest.raises(ValueError, match="GPU memory"):
+        m(torch.rand(4, 3))
+    with pytest.raises(RuntimeError, match="nr_feat_per_level"):
+        pe.PermutoEncoding(3, 64, 2, 4, [1.0, 0.5], device="cpu")
+    with pytest.raises(RuntimeError, match="pos_dim"):
+        pe.PermutoEncoding(9, 64, 2, 2, [1.0, 0.5], device="cpu")
+    with pytest.raises(ValueError, match="one entry per level"):
+        pe.PermutoEncoding(3, 64, 3, 2, [1.0, 0.5], device="cpu")
+    import permutohedral_encoding
+    assert permutohedral_encoding.PermutoEncoding is pe.PermutoEncoding
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "permutohedral_encoding_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")) or f == "Makefile":
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("oracle of", ""), f"{f} mentions the oracle"
+
+
+def test_workloads_are_seeded_and_shaped():
+    w = workloads.WORKLOADS["c3"].scaled(1000)
+    a, b = workloads.make_inputs(w), workloads.make_inputs(w)
+    for k in a:
+        assert np.array_equal(a[k], b[k])
+    assert a["pos"].shape == (1000, 4) and a["grad"].shape == (24, 2, 1000) and a["table"].shape == (24, 1 << 18, 2)
+    assert np.allclose(workloads.scale_list(w)[[0, -1]], [1.0, 1e-4])
+    s = workloads.make_inputs(workloads.WORKLOADS["c5"].scaled(4000), need=("pos",))["pos"]
+    r = np.linalg.norm(s - 0.5, axis=1)
+    assert abs(r.mean() - 0.5) < 5e-3 and 0.015 < r.std() < 0.025
+    assert workloads.WORKLOADS["c2"].point_levels == 25165824
