@@ -241,8 +241,8 @@ backward_pos_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
         const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
         const float* gp = grad_sliced + (static_cast<size_t>(level) * 2) * n_points + n;
-        const float g0 = gp[0] * w_level, g1 = gp[n_points] * w_level;
-        const fvec<D + 1> dB = v.f0 * g0 + v.f1 * g1;
+        const float g0 = gp[0], g1 = gp[n_points];
+        const fvec<D + 1> dB = (v.f0 * w_level) * g0 + (v.f1 * w_level) * g1;  // :688-689
         total += bary_grad_to_pos_grad<D>(s.rank, dB, sf);
     }
     float* o = positions_grad + static_cast<size_t>(n) * D;

@@ -213,6 +213,10 @@ __device__ __forceinline__ uvec<D + 1> vertex_hashes(ivec<D + 1> rank, uint32_t 
     return h;
 }
 
+// The three gradient chains below evaluate their sums in the same order, with the same
+// intermediate roundings, as the reference's loops, so that every term a kernel adds is the same
+// fp32 number the CPU checker computes; only the order of atomic accumulation can then differ.
+
 // d(loss)/d(barycentric) -> d(loss)/d(position) for one level (EncodingGPU.cuh:698-740).
 // dB[r] is the derivative w.r.t. the weight of vertex r.
 template <int D>
@@ -220,33 +224,39 @@ __device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<
                                                          const float* __restrict__ sf) {
     constexpr int D1 = D + 1;
     constexpr float kInv = 1.0f / D1;
-    // diff[m] = dB[D-m] - dB[D+1-m], with dB[D+1] = dB[0] (the wrap-around term, :698)
+    // dE[i] = dB[D-rank[i]]/(D+1) - dB[D+1-rank[i]]/(D+1), with dB[D+1] = dB[0] (the wrap-around
+    // term, :698).  As a function of the rank m: diff[m] = dB[D-m]/(D+1) - dB[D+1-m]/(D+1).
+    const fvec<D1> scaled = dB * kInv;
     fvec<D1> diff;
-    diff[0] = dB[D] - dB[0];
+    diff[0] = scaled[D] - scaled[0];
     static_for<D>(PENC_BODY(mm) {
         PENC_INDEX(mm);
         constexpr int m = mm + 1;
-        diff[m] = dB[D - m] - dB[D1 - m];
+        diff[m] = scaled[D - m] - scaled[D1 - m];
     });
-    // dE[i] = diff[rank[i]] / (D+1)
     fvec<D1> dE;
     static_for<D1>(PENC_BODY(i) {
         PENC_INDEX(i);
         float acc = diff[0];
         static_for<D>(PENC_BODY(mm) {
-        PENC_INDEX(mm);
+            PENC_INDEX(mm);
             constexpr int m = mm + 1;
             const float x = diff[m];
             acc = (rank[i] == m) ? x : acc;
         });
-        dE[i] = acc * kInv;
+        dE[i] = acc;
     });
+    // dP[i] = sum_{j<=i} dE[j]*sf[i] - dE[i+1]*sf[i]*(i+1)   (:729-740)
     fvec<D> dP;
-    float run = 0.0f;
     static_for<D>(PENC_BODY(i) {
         PENC_INDEX(i);
-        run += dE[i];
-        dP[i] = sf[i] * (run - static_cast<float>(i + 1) * dE[i + 1]);
+        float acc = dE[0] * sf[i];
+        static_for<i>(PENC_BODY(jj) {
+            PENC_INDEX(jj);
+            acc += dE[jj + 1] * sf[i];
+        });
+        acc -= dE[i + 1] * sf[i] * static_cast<float>(i + 1);
+        dP[i] = acc;
     });
     return dP;
 }
@@ -259,16 +269,21 @@ __device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_bary(ivec<D + 1> rank, f
     constexpr float kInv = 1.0f / D1;
     fvec<D> g;
     static_for<D>(PENC_BODY(i) {
-        PENC_INDEX(i); g[i] = q[i] * sf[i]; });
-    // dE[j] = sum_{i>=j} g[i] - j*g[j-1]
+        PENC_INDEX(i);
+        g[i] = q[i] * sf[i];
+    });
+    // dE[j] = g[j] + g[j+1] + ... + g[D-1] (summed in ascending order, :1187-1194), then
+    // dE[j] -= g[j-1]*j (:1196-1199)
     fvec<D1> dE;
-    float tail = 0.0f;
     dE[D] = 0.0f;
-    static_for<D>(PENC_BODY(k) {
-        PENC_INDEX(k);
-        constexpr int j = D - 1 - k;
-        tail += g[j];
-        dE[j] = tail;
+    static_for<D>(PENC_BODY(j) {
+        PENC_INDEX(j);
+        float acc = g[j];
+        static_for<D - 1 - j>(PENC_BODY(k) {
+            PENC_INDEX(k);
+            acc += g[j + 1 + k];
+        });
+        dE[j] = acc;
     });
     static_for<D>(PENC_BODY(jj) {
         PENC_INDEX(jj);
@@ -279,7 +294,7 @@ __device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_bary(ivec<D + 1> rank, f
     const fvec<D1> sorted = by_rank<D>(rank, dE);
     // dB[k] = sorted[D-k] - sorted[D+1-k]; dB[D+1] = -sorted[0] is folded into dB[0] (:1218)
     fvec<D1> dB;
-    dB[0] = sorted[D] - sorted[0];
+    dB[0] = sorted[D] + (0.0f - sorted[0]);
     static_for<D>(PENC_BODY(rr) {
         PENC_INDEX(rr);
         constexpr int r = rr + 1;
