@@ -115,6 +115,8 @@ def main():
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-probes", action="store_true", help="skip the memory-system probes")
+    ap.add_argument("--levels-per-pass", type=int, default=0,
+                    help="levels binned per scatter pass (0: library default, -1: no workspace, direct atomics)")
     ap.add_argument("--cpu-sample", type=int, default=1 << 18, help="points in the CPU baseline sample")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -156,15 +158,18 @@ def main():
                               P(win), P(out), 0, 1.0, stream)
         assert rc == 0, rc
 
+    ws_bytes = int(lib.penc_scatter_workspace_bytes(d, n, levels, cap, args.levels_per_pass)) if args.levels_per_pass >= 0 else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+
     def backward():
         rc = lib.penc_backward(d, 2, n, levels, cap, P(inp.m_positions_raw), P(inp.m_lattice_values), P(sf), P(shift),
-                               P(win), P(grad), P(tgrad) if want_table else None, P(pgrad), stream)
+                               P(win), P(grad), P(tgrad) if want_table else None, P(pgrad), P(ws), ws_bytes, stream)
         assert rc == 0, rc
 
     def double_backward():
         rc = lib.penc_double_backward_from_positions(d, 2, n, levels, cap, P(inp.m_positions_raw),
                                                      P(inp.m_lattice_values), P(sf), P(shift), P(win), P(dpos), P(grad),
-                                                     P(tgrad), P(ggs), 0, stream)
+                                                     P(tgrad), P(ggs), 0, P(ws), ws_bytes, stream)
         assert rc == 0, rc
 
     phases = [("forward", forward)]

@@ -23,6 +23,11 @@
  *                                             permuted view of [L][2][C], src/Encoding.cu:141,204)
  *        positions_grad       [N][D]         (the reference returns this logical shape as a
  *                                             transposed view of [D][N], src/Encoding.cu:152,205)
+ *  - `workspace` (optional, may be NULL) is device scratch memory of `workspace_bytes` bytes that
+ *    the table-gradient scatter uses to turn its random atomics into streaming traffic; its
+ *    contents on entry and exit are meaningless.  penc_scatter_workspace_bytes() suggests a size;
+ *    any size works (a small one means more passes, none means direct atomics).  Results do not
+ *    depend on it beyond the order of floating-point accumulation.
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is enqueued and
  *    the call returns without synchronising, like the reference's launches on the current stream.
  *  - D = pos_dim in 2..8, nr_feat must be 2 (reference: Encoding.cuh:139-156 supports 2..7 / 2).
@@ -31,6 +36,7 @@
 #ifndef PENC_H_
 #define PENC_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -56,6 +62,13 @@ int penc_extra_levels(int pos_dim, int nr_feat, int concat_points);
  * Replaces: EncodingFixedParams::compute_scale_factor_tensor, Encoding.cuh:55-69. */
 int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* scale_factor_out);
 
+/* Suggested size of the `workspace` argument of the two gradient calls below for binning
+ * `levels_per_pass` levels at a time (<= 0: the library's default); 0 when the capacity is too
+ * large for binning.  No counterpart in the reference (its scatter is one atomicAdd per value,
+ * EncodingGPU.cuh:409-410). */
+size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
+                                    int levels_per_pass);
+
 /* Slice: sliced_values[l][f][n] = sum over the D+1 simplex vertices of
  * lattice_values[l][slot][f] * barycentric * anneal_window[l]; extra levels copy
  * positions * points_scaling (zero-padded).
@@ -75,7 +88,7 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* positions, const float* lattice_values, const float* scale_factor,
                   const float* random_shift, const float* anneal_window,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
-                  void* stream);
+                  void* workspace, size_t workspace_bytes, void* stream);
 
 /* Double backward from d(loss)/d(positions_grad): gradient w.r.t. lattice_values and w.r.t.
  * grad_sliced_values ([L+E][2][N], zeros in the extra levels).  Either output may be NULL.
@@ -88,7 +101,8 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
                                         const float* random_shift, const float* anneal_window,
                                         const float* double_positions_grad,
                                         const float* grad_sliced_values, float* lattice_values_grad,
-                                        float* grad_grad_sliced_values, int concat_points, void* stream);
+                                        float* grad_grad_sliced_values, int concat_points, void* workspace,
+                                        size_t workspace_bytes, void* stream);
 
 /* Introspection for parity checks: what the kernels derive from each (level, point) before they
  * touch the table.  Outputs are [L][N][D+1]; each may be NULL.

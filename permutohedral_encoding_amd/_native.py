@@ -25,13 +25,15 @@ _SIGNATURES = {
     "penc_forward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                     _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                     ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
+    "penc_scatter_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                       ctypes.c_int]),
     "penc_backward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                      _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
-                                     ctypes.c_void_p]),
+                                     ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_double_backward_from_positions": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
                                                            ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int,
-                                                           ctypes.c_void_p]),
+                                                           ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
                                           _c_f32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, _c_f32p,
                                           ctypes.c_void_p]),
@@ -76,6 +78,21 @@ def scale_factors(pos_dim, sigmas):
     out = np.empty((sig.size, int(pos_dim)), np.float32)
     _check(lib().penc_scale_factors(int(pos_dim), int(sig.size), sig.ctypes.data, out.ctypes.data), "scale_factors")
     return out
+
+
+# Levels binned per pass by the table-gradient scatter (0: the library's default, < 0: no workspace,
+# i.e. direct atomics).  The workspace is taken from torch's caching allocator for the duration of a call.
+LEVELS_PER_PASS = 0
+
+
+def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device):
+    if LEVELS_PER_PASS < 0:
+        return None
+    nbytes = int(lib().penc_scatter_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels), int(capacity),
+                                                    int(LEVELS_PER_PASS)))
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
 def _ptr(t):
@@ -206,10 +223,11 @@ class EncodingWrapper:
         if lv_grad is None and pos_grad is None:
             return None, None
         with torch.cuda.device(pos.device):
+            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device) if lv_grad is not None else None
             _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
                                        _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
-                                       _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(pos_grad), _stream()),
-                   "backward")
+                                       _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(pos_grad),
+                                       _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
         return lv_grad, pos_grad
 
     def double_backward_from_positions(self, inp, double_positions_grad, grad_sliced_values_monolithic):
@@ -226,10 +244,12 @@ class EncodingWrapper:
         lv_grad = torch.empty_like(lv)
         ggs = torch.empty_like(grad_sliced_values_monolithic)
         with torch.cuda.device(pos.device):
+            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device)
             _check(lib().penc_double_backward_from_positions(
                 self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
                 _ptr(win), _ptr(dpos), _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(ggs),
-                int(fp.m_concat_points), _stream()), "double_backward_from_positions")
+                int(fp.m_concat_points), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
+                "double_backward_from_positions")
         return lv_grad, ggs
 
     def simplex_debug(self, positions, capacity):

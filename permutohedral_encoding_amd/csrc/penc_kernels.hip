@@ -22,12 +22,11 @@
 
 #include "../../include/penc.h"
 #include "penc_lattice.hpp"
+#include "penc_scatter.hpp"
 
 namespace penc {
 
-constexpr int kBlock = 256;         // 4 wavefronts
-constexpr int kCacheLines = 2048;   // LDS accumulate-cache lines per workgroup (tag + 2 floats = 24 KiB)
-constexpr int kTilesPerGroup = 16;  // point tiles a table-gradient workgroup walks before flushing
+constexpr int kDefaultLevelsPerPass = 4;  // levels binned per pass when the caller lets the library size the workspace
 
 __device__ __forceinline__ float2 load_vertex(const float* __restrict__ level_table, uint32_t slot) {
     return *reinterpret_cast<const float2*>(level_table + 2 * static_cast<size_t>(slot));
@@ -104,148 +103,40 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 }
 
 // ------------------------------------------------------------------------------------------
-// scatter-add into the table gradient with wave- and workgroup-level combining
-
-__device__ __forceinline__ void global_add(float* addr, float v) {
-    __hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Sum over the 64 lanes of a wavefront; the total is valid in lane 63.
-__device__ __forceinline__ float wave_sum_to_last_lane(float v) {
-    // row_shr:1,2,4,8 build the total of each row of 16 in its last lane (lanes shifted in from
-    // outside the row read 0); row_bcast:15 adds it into rows 1 and 3, row_bcast:31 into rows 2 and 3
-    constexpr int kShr1 = 0x111, kShr2 = 0x112, kShr4 = 0x114, kShr8 = 0x118, kBcast15 = 0x142, kBcast31 = 0x143;
-#define PENC_DPP_ADD(CTRL, ROW_MASK) \
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true))
-    PENC_DPP_ADD(kShr1, 0xf);
-    PENC_DPP_ADD(kShr2, 0xf);
-    PENC_DPP_ADD(kShr4, 0xf);
-    PENC_DPP_ADD(kShr8, 0xf);
-    PENC_DPP_ADD(kBcast15, 0xa);
-    PENC_DPP_ADD(kBcast31, 0xc);
-#undef PENC_DPP_ADD
-    return v;
-}
-
-struct AccumCache {
-    int tag[kCacheLines];
-    float val[kCacheLines][2];
-};
-
-__device__ __forceinline__ void cache_clear(AccumCache& c) {
-    for (int e = threadIdx.x; e < kCacheLines; e += kBlock) {
-        c.tag[e] = -1;
-        c.val[e][0] = 0.0f;
-        c.val[e][1] = 0.0f;
-    }
-}
-
-// Global fp32 atomics are serviced per 64-byte segment touched by a wave instruction, whatever
-// the number of lanes in it (measured: 21 G segments/s, from 1 to 16 lanes per segment), so the two
-// features of a slot, which are adjacent in memory, should leave in ONE instruction.  Lanes are
-// paired (2p, 2p+1): first both lanes of a pair add the two features of the even lane's slot, then
-// those of the odd lane's slot.  Must be called with all 64 lanes of the wave active.
-__device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad, bool need, uint32_t slot,
-                                                 float a0, float a1) {
-    constexpr int kFromEven = 0xA0;  // quad_perm:[0,0,2,2]
-    constexpr int kFromOdd = 0xF5;   // quad_perm:[1,1,3,3]
-    const int odd = threadIdx.x & 1;
-    const int slot_i = static_cast<int>(slot), need_i = need ? 1 : 0;
-    const int a0_i = __builtin_bit_cast(int, a0), a1_i = __builtin_bit_cast(int, a1);
-    {   // the even lane's contribution: even lane adds feature 0, odd lane feature 1
-        const int s = __builtin_amdgcn_update_dpp(0, slot_i, kFromEven, 0xf, 0xf, true);
-        const int n = __builtin_amdgcn_update_dpp(0, need_i, kFromEven, 0xf, 0xf, true);
-        const int hi = __builtin_amdgcn_update_dpp(0, a1_i, kFromEven, 0xf, 0xf, true);
-        const float v = __builtin_bit_cast(float, odd ? hi : a0_i);
-        if (n) global_add(level_grad + 2 * static_cast<size_t>(static_cast<uint32_t>(s)) + odd, v);
-    }
-    {   // the odd lane's contribution
-        const int s = __builtin_amdgcn_update_dpp(0, slot_i, kFromOdd, 0xf, 0xf, true);
-        const int n = __builtin_amdgcn_update_dpp(0, need_i, kFromOdd, 0xf, 0xf, true);
-        const int lo = __builtin_amdgcn_update_dpp(0, a0_i, kFromOdd, 0xf, 0xf, true);
-        const float v = __builtin_bit_cast(float, odd ? a1_i : lo);
-        if (n) global_add(level_grad + 2 * static_cast<size_t>(static_cast<uint32_t>(s)) + odd, v);
-    }
-}
-
-// Adds (a0, a1) to slot `slot` of this level's gradient slice.  `active` is false for lanes that
-// carry no point (tail of the last tile); they take part in the wave-wide steps only.
-// Must be called with all 64 lanes of the wave active.
-__device__ __forceinline__ void cache_add(AccumCache& c, float* __restrict__ level_grad, bool active,
-                                          uint32_t slot, float a0, float a1) {
-    // wave-uniform slot: one DPP reduction, one lane adds
-    const uint32_t first = __builtin_amdgcn_readfirstlane(slot);
-    if (__all(active && slot == first)) {
-        a0 = wave_sum_to_last_lane(a0);
-        a1 = wave_sum_to_last_lane(a1);
-        active = (threadIdx.x & 63) == 63;
-    }
-    bool need_global = false;
-    if (active) {
-        const int e = static_cast<int>(slot & (kCacheLines - 1));
-        int owner = c.tag[e];
-        if (owner == -1) {
-            owner = atomicCAS(&c.tag[e], -1, static_cast<int>(slot));
-            if (owner == -1) owner = static_cast<int>(slot);
-        }
-        if (owner == static_cast<int>(slot)) {
-            __hip_atomic_fetch_add(&c.val[e][0], a0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            __hip_atomic_fetch_add(&c.val[e][1], a1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        } else {
-            need_global = true;
-        }
-    }
-    global_add_pairs(level_grad, need_global, slot, a0, a1);
-}
-
-__device__ __forceinline__ void cache_flush(AccumCache& c, float* __restrict__ level_grad) {
-    for (int e = threadIdx.x; e < kCacheLines; e += kBlock) {
-        const int owner = c.tag[e];
-        if (owner != -1) {
-            float* g = level_grad + 2 * static_cast<size_t>(owner);
-            global_add(g, c.val[e][0]);
-            global_add(g + 1, c.val[e][1]);
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
 // backward w.r.t. the table (EncodingGPU.cuh:259-414)
 
 template <int D>
-__global__ void __launch_bounds__(kBlock)
-backward_table_kernel(int n_points, uint32_t capacity, uint32_t cap_mask,
+__global__ void __launch_bounds__(kScatterBlock)
+backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
-                      const float* __restrict__ grad_sliced, float* __restrict__ table_grad) {
-    __shared__ AccumCache cache;
-    const int level = blockIdx.y;
+                      const float* __restrict__ grad_sliced, float* __restrict__ table_grad, BinTarget pass_bins) {
+    __shared__ ScatterState state;
+    const int level = first_level + blockIdx.y;
     const float w_level = window[level];
     if (w_level == 0.0f) return;
-    cache_clear(cache);
-    __syncthreads();
+    scatter_begin(state);
+    const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
     float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
-    const int first_tile = blockIdx.x * kTilesPerGroup;
-    for (int t = 0; t < kTilesPerGroup; ++t) {
-        const int tile_base = (first_tile + t) * kBlock;
+    for (int t = 0; t < kScatterTiles; ++t) {
+        const int64_t tile_base = (static_cast<int64_t>(blockIdx.x) * kScatterTiles + t) * kScatterBlock;
         if (tile_base >= n_points) break;
-        const int n = tile_base + threadIdx.x;
-        const bool active = n < n_points;
-        const int nn = active ? n : n_points - 1;
+        const bool active = tile_base + threadIdx.x < n_points;
+        const int nn = active ? static_cast<int>(tile_base) + threadIdx.x : n_points - 1;
         const float g0 = g0p[nn], g1 = g1p[nn];
         const Located<D> s = locate<D>(load_point<D>(positions, nn), random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
-        const fvec<D + 1> w = barycentric<D>(s.rank, s.delta);
+        const fvec<D + 1> w = barycentric<D>(s.rank, s.delta) * w_level;
+        uvec<D + 1> slot;
         static_for<D + 1>(PENC_BODY(r) {
-        PENC_INDEX(r);
-            const float wr = w[r] * w_level;
-            cache_add(cache, level_grad, active, to_slot(h[r], capacity, cap_mask), g0 * wr, g1 * wr);
+            PENC_INDEX(r);
+            slot[r] = to_slot(h[r], capacity, cap_mask);
         });
+        scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
     }
-    __syncthreads();
-    cache_flush(cache, level_grad);
+    scatter_end(state, level_grad, bins, blockIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -284,58 +175,57 @@ backward_pos_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_
 // (EncodingGPU.cuh:1016-1257 scatter into the table gradient, 1260-1493 grad of grad_sliced)
 
 template <int D, bool kTableGrad, bool kGradGrad>
-__global__ void __launch_bounds__(kBlock)
-double_backward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
+__global__ void __launch_bounds__(kScatterBlock)
+double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t capacity, uint32_t cap_mask,
                        const float* __restrict__ positions, const float* __restrict__ table,
                        const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                        const float* __restrict__ window, const float* __restrict__ double_pos_grad,
                        const float* __restrict__ grad_sliced, float* __restrict__ table_grad,
-                       float* __restrict__ grad_grad_sliced) {
-    __shared__ AccumCache cache;
-    const int level = blockIdx.y;
+                       float* __restrict__ grad_grad_sliced, BinTarget pass_bins) {
+    __shared__ ScatterState state;
+    const int level = first_level + blockIdx.y;
     const bool extra_level = level >= n_levels;  // concat levels: zeros (:1290-1295)
     const float w_level = extra_level ? 0.0f : window[level];
     const bool live = w_level != 0.0f;
     if (!live && !kGradGrad) return;
-    if (kTableGrad && live) {
-        cache_clear(cache);
-        __syncthreads();
-    }
+    if (kTableGrad && live) scatter_begin(state);
     const int lvl = extra_level ? 0 : level;
+    const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
     float* level_grad = kTableGrad ? table_grad + static_cast<size_t>(lvl) * capacity * 2 : nullptr;
     const float* level_table = table + static_cast<size_t>(lvl) * capacity * 2;
     const float* sf = scale_factor + lvl * D;
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
-    const int first_tile = blockIdx.x * kTilesPerGroup;
-    for (int t = 0; t < kTilesPerGroup; ++t) {
-        const int tile_base = (first_tile + t) * kBlock;
+    for (int t = 0; t < kScatterTiles; ++t) {
+        const int64_t tile_base = (static_cast<int64_t>(blockIdx.x) * kScatterTiles + t) * kScatterBlock;
         if (tile_base >= n_points) break;
-        const int n = tile_base + threadIdx.x;
-        const bool active = n < n_points;
+        const bool active = tile_base + threadIdx.x < n_points;
+        const int n = static_cast<int>(tile_base) + threadIdx.x;
         const int nn = active ? n : n_points - 1;
         float gg0 = 0.0f, gg1 = 0.0f;
         if (live) {
             const Located<D> s = locate<D>(load_point<D>(positions, nn), random_shift + lvl * D, sf);
             const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
+            uvec<D + 1> slot;
+            static_for<D + 1>(PENC_BODY(r) {
+                PENC_INDEX(r);
+                slot[r] = to_slot(h[r], capacity, cap_mask);
+            });
             Vertices<D> v;
             if constexpr (kGradGrad) v = load_vertices<D>(level_table, h, capacity, cap_mask);
-            const fvec<D + 1> dB = pos_grad_grad_to_bary<D>(s.rank, load_point<D>(double_pos_grad, nn), sf);
-            float g0 = 0.0f, g1 = 0.0f;
-            if constexpr (kTableGrad) {
-                g0 = g0p[nn];
-                g1 = g1p[nn];
+            // dB[r] * w_level, then times g_f or times the vertex value (:1244-1245, :1484-1485)
+            const fvec<D + 1> wr = pos_grad_grad_to_bary<D>(s.rank, load_point<D>(double_pos_grad, nn), sf) * w_level;
+            if constexpr (kGradGrad) {
+                static_for<D + 1>(PENC_BODY(r) {
+                    PENC_INDEX(r);
+                    gg0 += wr[r] * v.f0[r];
+                    gg1 += wr[r] * v.f1[r];
+                });
             }
-            static_for<D + 1>(PENC_BODY(r) {
-        PENC_INDEX(r);
-                const float wr = dB[r] * w_level;
-                if constexpr (kGradGrad) {
-                    gg0 += wr * v.f0[r];
-                    gg1 += wr * v.f1[r];
-                }
-                if constexpr (kTableGrad)
-                    cache_add(cache, level_grad, active, to_slot(h[r], capacity, cap_mask), wr * g0, wr * g1);
-            });
+            if constexpr (kTableGrad) {
+                const float g0 = g0p[nn], g1 = g1p[nn];
+                scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, slot, wr * g0, wr * g1);
+            }
         }
         if (kGradGrad && active) {
             float* o = grad_grad_sliced + (static_cast<size_t>(level) * 2) * n_points + n;
@@ -343,10 +233,7 @@ double_backward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t c
             o[n_points] = gg1;
         }
     }
-    if (kTableGrad && live) {
-        __syncthreads();
-        cache_flush(cache, level_grad);
-    }
+    if (kTableGrad && live) scatter_end(state, level_grad, bins, blockIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -414,6 +301,69 @@ inline int clear_table_grad(float* g, int levels, int capacity, hipStream_t st) 
     return check_launch();
 }
 
+// How a workspace is cut into slot-range bins (see penc_scatter.hpp).  The levels are processed in
+// passes of `levels_per_pass`; every pass reuses the same bins, so a smaller workspace means more,
+// shorter passes (whose records are more likely still in cache when they are read back), not less
+// binning.
+struct BinPlan {
+    bool enabled = false;
+    int levels_per_pass = 0;
+    BinTarget target{};
+};
+
+inline uint32_t bins_for_capacity(int capacity) {
+    return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
+}
+
+inline unsigned scatter_groups(int64_t n) { return static_cast<unsigned>((n + kGroupPoints - 1) / kGroupPoints); }
+
+// Records one scattering workgroup may leave in one bin: its share of the group's
+// kGroupPoints*(D+1) contributions plus the flushed cache lines, with three standard deviations
+// of a uniform hash on top.  A segment that still overflows spills to direct atomics.
+inline uint32_t wanted_segment_capacity(int pos_dim, uint32_t n_bins) {
+    const double mean = (static_cast<double>(kGroupPoints) * (pos_dim + 1) + kCacheLines) / n_bins;
+    return static_cast<uint32_t>(mean + 3.0 * __builtin_sqrt(mean) + 8.0);
+}
+
+inline size_t bin_bytes_per_level(uint32_t n_bins, uint32_t n_groups, uint32_t segment_capacity) {
+    const size_t segments = static_cast<size_t>(n_bins) * n_groups;
+    return segments * (sizeof(uint32_t) + static_cast<size_t>(segment_capacity) * sizeof(BinRecord));
+}
+
+inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, void* workspace, size_t bytes) {
+    BinPlan p;
+    const uint32_t n_bins = bins_for_capacity(capacity);
+    const uint32_t n_groups = scatter_groups(n);
+    if (workspace == nullptr || n_bins > static_cast<uint32_t>(kMaxBins)) return p;
+    const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
+    const size_t lost = base - reinterpret_cast<uintptr_t>(workspace);
+    if (bytes < lost + 4096) return p;
+    bytes -= lost + 256;
+    const size_t segments = static_cast<size_t>(n_bins) * n_groups;
+    uint32_t cap = wanted_segment_capacity(pos_dim, n_bins);
+    if (bytes < bin_bytes_per_level(n_bins, n_groups, cap)) {  // not even one level at the wanted size: shrink the segments
+        if (bytes < segments * (sizeof(uint32_t) + 16 * sizeof(BinRecord))) return p;
+        cap = static_cast<uint32_t>((bytes / segments - sizeof(uint32_t)) / sizeof(BinRecord));
+    }
+    const size_t fit = bytes / bin_bytes_per_level(n_bins, n_groups, cap);
+    p.levels_per_pass = static_cast<int>(fit < static_cast<size_t>(levels) ? fit : static_cast<size_t>(levels));
+    p.target.n_bins = n_bins;
+    p.target.n_groups = n_groups;
+    p.target.segment_capacity = cap;
+    p.target.counts = reinterpret_cast<uint32_t*>(base);
+    const size_t counts_bytes = (static_cast<size_t>(p.levels_per_pass) * segments * sizeof(uint32_t) + 255u) & ~size_t{255};
+    p.target.records = reinterpret_cast<BinRecord*>(base + counts_bytes);
+    p.enabled = true;
+    return p;
+}
+
+inline int reduce_bins(const BinPlan& p, const float* window, int first_level, int n_levels_in_pass, int capacity,
+                       float* table_grad, hipStream_t st) {
+    hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass, kReduceSplit), dim3(kReduceBlock), 0, st,
+                       p.target, window, static_cast<uint32_t>(capacity), table_grad, first_level);
+    return check_launch();
+}
+
 #define PENC_DISPATCH_D(D_, ...)                                  \
     switch (D_) {                                                  \
         case 2: { constexpr int DD = 2; __VA_ARGS__; } break;      \
@@ -427,7 +377,6 @@ inline int clear_table_grad(float* g, int levels, int capacity, hipStream_t st) 
     }
 
 inline unsigned tiles(int64_t n) { return static_cast<unsigned>((n + kBlock - 1) / kBlock); }
-inline unsigned tile_groups(int64_t n) { return (tiles(n) + kTilesPerGroup - 1) / kTilesPerGroup; }
 
 }  // namespace penc
 
@@ -451,6 +400,16 @@ const char* penc_status_string(int status) {
 int penc_extra_levels(int pos_dim, int nr_feat, int concat_points) {
     if (!concat_points || nr_feat <= 0) return 0;
     return (pos_dim + nr_feat - 1) / nr_feat;
+}
+
+size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, int levels_per_pass) {
+    if (pos_dim < 2 || pos_dim > 8 || nr_positions <= 0 || nr_levels <= 0 || capacity <= 0) return 0;
+    const uint32_t n_bins = bins_for_capacity(capacity);
+    if (n_bins > static_cast<uint32_t>(kMaxBins)) return 0;
+    if (levels_per_pass <= 0) levels_per_pass = kDefaultLevelsPerPass;
+    if (levels_per_pass > nr_levels) levels_per_pass = nr_levels;
+    const size_t per_level = bin_bytes_per_level(n_bins, scatter_groups(nr_positions), wanted_segment_capacity(pos_dim, n_bins));
+    return per_level * static_cast<size_t>(levels_per_pass) + 1024;
 }
 
 int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* scale_factor_out) {
@@ -487,7 +446,7 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* positions, const float* lattice_values, const float* scale_factor,
                   const float* random_shift, const float* anneal_window,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
-                  void* stream) {
+                  void* workspace, size_t workspace_bytes, void* stream) {
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
     if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_sliced_values)
         return PENC_ERR_NULL_POINTER;
@@ -499,11 +458,19 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     if (lattice_values_grad) {
         if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-        const dim3 grid(tile_groups(nr_positions), nr_levels);
-        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD>), grid, dim3(kBlock), 0, st, n, cap, mask,
-                                                    positions, scale_factor, random_shift, anneal_window,
-                                                    grad_sliced_values, lattice_values_grad));
-        if (int rc = check_launch()) return rc;
+        const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, workspace, workspace_bytes);
+        const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
+        for (int first = 0; first < nr_levels; first += per_pass) {
+            const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
+            const dim3 grid(scatter_groups(nr_positions), count);
+            PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD>), grid, dim3(kScatterBlock), 0, st, n,
+                                                        first, cap, mask, positions, scale_factor, random_shift,
+                                                        anneal_window, grad_sliced_values, lattice_values_grad,
+                                                        plan.target));
+            if (int rc = check_launch()) return rc;
+            if (plan.enabled)
+                if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, lattice_values_grad, st)) return rc;
+        }
     }
     if (positions_grad) {
         PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions)), dim3(kBlock), 0,
@@ -521,7 +488,8 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
                                         const float* random_shift, const float* anneal_window,
                                         const float* double_positions_grad,
                                         const float* grad_sliced_values, float* lattice_values_grad,
-                                        float* grad_grad_sliced_values, int concat_points, void* stream) {
+                                        float* grad_grad_sliced_values, int concat_points, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
     const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
     if (!positions || !lattice_values || !scale_factor || !random_shift || !anneal_window ||
@@ -532,24 +500,36 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
-    if (lattice_values_grad)
-        if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-    const dim3 block(kBlock);
-#define PENC_LAUNCH_DB(TG, GG, LEVELS)                                                                           \
+    const dim3 block(kScatterBlock);
+#define PENC_LAUNCH_DB(TG, GG, FIRST, COUNT, TARGET)                                                             \
     PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((double_backward_kernel<DD, TG, GG>),                            \
-                                                dim3(tile_groups(nr_positions), LEVELS), block, 0, st, n, nr_levels, \
-                                                cap, mask, positions, lattice_values, scale_factor, random_shift, \
-                                                anneal_window, double_positions_grad, grad_sliced_values,        \
-                                                lattice_values_grad, grad_grad_sliced_values))
-    if (lattice_values_grad && grad_grad_sliced_values) {
-        PENC_LAUNCH_DB(true, true, nr_levels + extra);
-    } else if (lattice_values_grad) {
-        PENC_LAUNCH_DB(true, false, nr_levels);
-    } else {
-        PENC_LAUNCH_DB(false, true, nr_levels + extra);
+                                                dim3(scatter_groups(nr_positions), COUNT), block, 0, st, n, nr_levels, \
+                                                FIRST, cap, mask, positions, lattice_values, scale_factor,        \
+                                                random_shift, anneal_window, double_positions_grad,              \
+                                                grad_sliced_values, lattice_values_grad, grad_grad_sliced_values, \
+                                                TARGET))
+    if (!lattice_values_grad) {
+        PENC_LAUNCH_DB(false, true, 0, nr_levels + extra, BinTarget{});
+        return check_launch();
+    }
+    if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
+    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, workspace, workspace_bytes);
+    const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
+    for (int first = 0; first < nr_levels; first += per_pass) {
+        int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
+        const int scatter_levels = count;
+        if (first + count == nr_levels && grad_grad_sliced_values) count += extra;  // the zero-filled concat levels
+        if (grad_grad_sliced_values) {
+            PENC_LAUNCH_DB(true, true, first, count, plan.target);
+        } else {
+            PENC_LAUNCH_DB(true, false, first, count, plan.target);
+        }
+        if (int rc = check_launch()) return rc;
+        if (plan.enabled)
+            if (int rc = reduce_bins(plan, anneal_window, first, scatter_levels, capacity, lattice_values_grad, st)) return rc;
     }
 #undef PENC_LAUNCH_DB
-    return check_launch();
+    return PENC_OK;
 }
 
 int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,

@@ -1,0 +1,266 @@
+// Scatter-add of (slot, value pair) contributions into one level's slice of the table gradient.
+//
+// What the memory system of gfx950 gives (measured with purpose-built probes):
+//   * a global fp32 atomic costs one request per 64-byte segment touched by a wave instruction,
+//     whatever the number of lanes in the segment (1..16), the scope or the footprint; the chip
+//     retires about 21 G such requests/s.  A level with many distinct slots is therefore bound
+//     by requests, not bytes.
+//   * ds_add_f32 retires about one lane every 3 clocks per CU, 30 times slower than integer LDS
+//     atomics (ds_add_u32, ds_cmpst_b32/b64) and than plain LDS reads and writes.
+//
+// Hence three stages, each taking what the previous one could not combine:
+//   1. Accumulate cache in LDS.  Every workgroup keeps a small open-addressed table
+//      (tag = slot) for the level it works on.  Coarse levels, where thousands of points share
+//      a handful of vertices, are absorbed here completely; the table is flushed once at the end.
+//   2. Slot-range bins (optional, needs a workspace).  A contribution that finds no line in the
+//      cache is appended, as a 12-byte record, to the bin of its slot range (each workgroup has a
+//      private segment in every bin, so appending costs one LDS counter increment and one
+//      store); a second kernel (bin_reduce_kernel) reads each bin back coalesced, sums it in
+//      LDS, and adds the range into the gradient with dense atomics (8 slots per request).  This
+//      turns the random scatter of the fine levels into streaming traffic.
+//   3. Direct global atomics, with the two features of a slot in one instruction (lane pairs),
+//      for whatever is left: no workspace, capacity too large for binning, or a full bin.
+// The result never depends on a stage hitting: every stage falls through to the next.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "penc_lattice.hpp"
+
+namespace penc {
+
+constexpr int kBlock = 256;            // threads per workgroup of the gather-type kernels (4 wavefronts)
+constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wavefronts share one accumulate cache)
+constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
+constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
+constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
+constexpr int kBinSlotsLog2 = 12;      // slots per bin: 4096 (32 KiB of sums in LDS)
+constexpr int kBinSlots = 1 << kBinSlotsLog2;
+constexpr int kMaxBins = 256;          // bins per level; capacities above kMaxBins*kBinSlots are not binned
+constexpr int kReduceBlock = 512;      // threads of a bin_reduce_kernel workgroup
+constexpr int kReduceSplit = 4;        // workgroups that share one bin in bin_reduce_kernel
+
+struct BinRecord {
+    uint32_t slot_in_bin;
+    float a0, a1;
+};
+
+// Where the misses of the levels of one launch go.  Every scattering workgroup (a "group" of
+// kGroupPoints points at one level) owns a private segment of `segment_capacity` records in every
+// bin, so appending needs no global atomics and no synchronisation: the cursor is an LDS counter.
+//   records [level_in_pass][bin][group][segment_capacity]
+//   counts  [level_in_pass][bin][group]            records actually written (<= segment_capacity)
+// `records` == nullptr disables binning.
+struct BinTarget {
+    BinRecord* records;
+    uint32_t* counts;
+    uint32_t n_bins;
+    uint32_t n_groups;
+    uint32_t segment_capacity;
+};
+
+// `pass` describes the first level of a launch; level k of the launch follows k bin arrays later.
+__device__ __forceinline__ BinTarget bins_of_level(const BinTarget& pass, uint32_t k) {
+    BinTarget t = pass;
+    if (pass.records != nullptr) {
+        const size_t segments = static_cast<size_t>(k) * pass.n_bins * pass.n_groups;
+        t.records += segments * pass.segment_capacity;
+        t.counts += segments;
+    }
+    return t;
+}
+
+__device__ __forceinline__ void global_add(float* addr, float v) {
+    __hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Sum over the 64 lanes of a wavefront; the total is valid in lane 63.
+__device__ __forceinline__ float wave_sum_to_last_lane(float v) {
+    // row_shr:1,2,4,8 build the total of each row of 16 in its last lane (lanes shifted in from
+    // outside the row read 0); row_bcast:15 adds it into rows 1 and 3, row_bcast:31 into rows 2 and 3
+    constexpr int kShr1 = 0x111, kShr2 = 0x112, kShr4 = 0x114, kShr8 = 0x118, kBcast15 = 0x142, kBcast31 = 0x143;
+#define PENC_DPP_ADD(CTRL, ROW_MASK) \
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true))
+    PENC_DPP_ADD(kShr1, 0xf);
+    PENC_DPP_ADD(kShr2, 0xf);
+    PENC_DPP_ADD(kShr4, 0xf);
+    PENC_DPP_ADD(kShr8, 0xf);
+    PENC_DPP_ADD(kBcast15, 0xa);
+    PENC_DPP_ADD(kBcast31, 0xc);
+#undef PENC_DPP_ADD
+    return v;
+}
+
+// Stage 3.  Lanes are paired (2p, 2p+1): first both lanes of a pair add the two features of the
+// even lane's slot, then those of the odd lane's slot, so that each 8-byte slot is one request.
+// Must be called with all 64 lanes of the wave active.
+__device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad, bool need, uint32_t slot,
+                                                 float a0, float a1) {
+    constexpr int kFromEven = 0xA0;  // quad_perm:[0,0,2,2]
+    constexpr int kFromOdd = 0xF5;   // quad_perm:[1,1,3,3]
+    const int odd = threadIdx.x & 1;
+    const int slot_i = static_cast<int>(slot), need_i = need ? 1 : 0;
+    const int a0_i = __builtin_bit_cast(int, a0), a1_i = __builtin_bit_cast(int, a1);
+    {   // the even lane's contribution: even lane adds feature 0, odd lane feature 1
+        const int s = __builtin_amdgcn_update_dpp(0, slot_i, kFromEven, 0xf, 0xf, true);
+        const int n = __builtin_amdgcn_update_dpp(0, need_i, kFromEven, 0xf, 0xf, true);
+        const int hi = __builtin_amdgcn_update_dpp(0, a1_i, kFromEven, 0xf, 0xf, true);
+        const float v = __builtin_bit_cast(float, odd ? hi : a0_i);
+        if (n) global_add(level_grad + 2 * static_cast<size_t>(static_cast<uint32_t>(s)) + odd, v);
+    }
+    {   // the odd lane's contribution
+        const int s = __builtin_amdgcn_update_dpp(0, slot_i, kFromOdd, 0xf, 0xf, true);
+        const int n = __builtin_amdgcn_update_dpp(0, need_i, kFromOdd, 0xf, 0xf, true);
+        const int lo = __builtin_amdgcn_update_dpp(0, a0_i, kFromOdd, 0xf, 0xf, true);
+        const float v = __builtin_bit_cast(float, odd ? a1_i : lo);
+        if (n) global_add(level_grad + 2 * static_cast<size_t>(static_cast<uint32_t>(s)) + odd, v);
+    }
+}
+
+// LDS state of a scattering workgroup.
+struct ScatterState {
+    int tag[kCacheLines];
+    float val[kCacheLines][2];
+    uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
+};
+
+__device__ __forceinline__ void scatter_begin(ScatterState& c) {
+    for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
+        c.tag[e] = -1;
+        c.val[e][0] = 0.0f;
+        c.val[e][1] = 0.0f;
+    }
+    for (int b = threadIdx.x; b < kMaxBins; b += kScatterBlock) c.bin_count[b] = 0u;
+    __syncthreads();
+}
+
+// Stage 2 for one contribution: append a record to this workgroup's segment of the slot's bin.
+// Returns false when the segment is full.
+__device__ __forceinline__ bool append_record(ScatterState& c, const BinTarget& bins, uint32_t group, uint32_t slot,
+                                              float a0, float a1) {
+    const uint32_t b = slot >> kBinSlotsLog2;
+    const uint32_t pos = atomicAdd(&c.bin_count[b], 1u);
+    if (pos >= bins.segment_capacity) return false;
+    BinRecord rec;
+    rec.slot_in_bin = slot & (kBinSlots - 1);
+    rec.a0 = a0;
+    rec.a1 = a1;
+    bins.records[(static_cast<size_t>(b) * bins.n_groups + group) * bins.segment_capacity + pos] = rec;
+    return true;
+}
+
+// One tile's D+1 contributions per thread through stages 1-3.  All 64 lanes of every wave must
+// call it together; `active` is false for lanes that carry no point (tail of the last tile), which
+// only take part in the wave-wide steps.
+template <int D>
+__device__ __forceinline__ void scatter_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+                                             uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
+                                             fvec<D + 1> a1) {
+    static_for<D + 1>(PENC_BODY(r) {
+        PENC_INDEX(r);
+        // stage 1; a wave whose lanes all hit one slot reduces with DPP and lets lane 63 add the sum
+        const uint32_t first = __builtin_amdgcn_readfirstlane(slot[r]);
+        float x0 = a0[r], x1 = a1[r];
+        bool act = active;
+        if (__all(active && slot[r] == first)) {
+            x0 = wave_sum_to_last_lane(x0);
+            x1 = wave_sum_to_last_lane(x1);
+            act = (threadIdx.x & 63) == 63;
+        }
+        bool miss = false;
+        if (act) {
+            const int e = static_cast<int>(slot[r] & (kCacheLines - 1));
+            int owner = c.tag[e];
+            if (owner == -1) {
+                owner = atomicCAS(&c.tag[e], -1, static_cast<int>(slot[r]));
+                if (owner == -1) owner = static_cast<int>(slot[r]);
+            }
+            if (owner == static_cast<int>(slot[r])) {
+                __hip_atomic_fetch_add(&c.val[e][0], x0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&c.val[e][1], x1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            } else {
+                miss = true;
+            }
+        }
+        // stage 2, then stage 3 for what stage 2 could not take
+        if (miss && bins.records != nullptr) miss = !append_record(c, bins, group, slot[r], x0, x1);
+        if (__any(miss)) global_add_pairs(level_grad, miss, slot[r], x0, x1);
+    });
+}
+
+// After the last tile: flushes the accumulate cache (through the bins when there are any) and
+// publishes how many records this workgroup left in each bin.  Call once, by all threads.
+__device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+                                            uint32_t group) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
+        const int owner = c.tag[e];
+        if (owner != -1) {
+            const float v0 = c.val[e][0], v1 = c.val[e][1];
+            const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
+            if (!binned) {
+                float* g = level_grad + 2 * static_cast<size_t>(owner);
+                global_add(g, v0);
+                global_add(g + 1, v1);
+            }
+        }
+    }
+    if (bins.records == nullptr) return;
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < bins.n_bins; b += kScatterBlock) {
+        const uint32_t n = c.bin_count[b];
+        bins.counts[static_cast<size_t>(b) * bins.n_groups + group] = n < bins.segment_capacity ? n : bins.segment_capacity;
+    }
+}
+
+// Second kernel of stage 2: kReduceSplit workgroups per (bin, level) sum the bin's records in LDS
+// and add the bin's slot range into the gradient.  Sums are kept as two floats packed in 64 bits
+// and updated with a compare-and-swap loop (ds_cmpst_rtn_b64), which runs at integer-atomic speed.
+// Each wavefront takes whole segments (one per scattering workgroup), so its loads are contiguous.
+__global__ void __launch_bounds__(kReduceBlock)
+bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity,
+                  float* __restrict__ table_grad, int first_level) {
+    __shared__ unsigned long long acc[kBinSlots];
+    const uint32_t bin = blockIdx.x;
+    const int level = first_level + blockIdx.y;
+    if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
+    const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
+    for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) acc[s] = 0ull;
+    __syncthreads();
+    constexpr uint32_t kWaves = kReduceBlock / 64;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
+    const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
+    for (uint32_t g = blockIdx.z * kWaves + wave; g < bins.n_groups; g += kWaves * kReduceSplit) {
+        const uint32_t count = counts[g];
+        const BinRecord* seg = recs + static_cast<size_t>(g) * bins.segment_capacity;
+        for (uint32_t i = lane; i < count; i += 64) {
+            const BinRecord rec = seg[i];
+            unsigned long long* cell = &acc[rec.slot_in_bin];
+            unsigned long long seen = *cell;
+            for (;;) {
+                const float s0 = __builtin_bit_cast(float, static_cast<uint32_t>(seen)) + rec.a0;
+                const float s1 = __builtin_bit_cast(float, static_cast<uint32_t>(seen >> 32)) + rec.a1;
+                const unsigned long long want = static_cast<unsigned long long>(__builtin_bit_cast(uint32_t, s0)) |
+                                                (static_cast<unsigned long long>(__builtin_bit_cast(uint32_t, s1)) << 32);
+                const unsigned long long got = atomicCAS(cell, seen, want);
+                if (got == seen) break;
+                seen = got;
+            }
+        }
+    }
+    __syncthreads();
+    float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
+    const uint32_t slot0 = bin << kBinSlotsLog2;
+    for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
+        const unsigned long long v = acc[s];
+        if (v != 0ull && slot0 + s < capacity) {
+            float* g = level_grad + 2 * static_cast<size_t>(slot0 + s);
+            global_add(g, __builtin_bit_cast(float, static_cast<uint32_t>(v)));
+            global_add(g + 1, __builtin_bit_cast(float, static_cast<uint32_t>(v >> 32)));
+        }
+    }
+}
+
+}  // namespace penc

@@ -271,3 +271,65 @@ def test_full_size_constant_table_gives_window():
     out = enc.forward(_native.EncodingInput(table, to_gpu(p["pos"]), win, False, False))
     assert torch.allclose(out[:, 0], (2.0 * win)[:, None].expand(-1, w.nr_points), rtol=1e-5)
     assert torch.allclose(out[:, 1], (-3.0 * win)[:, None].expand(-1, w.nr_points), rtol=1e-5)
+
+
+# ----------------------------------------------------------------------------- scatter workspace
+
+def _table_grads_with_workspace(enc, p, ws_bytes, d, cap, dpos=None):
+    """Calls the C ABI directly with a workspace of the given size (None: no workspace)."""
+    from permutohedral_encoding_amd import _native
+    lib = _native.lib()
+    fp = enc.fixed_params
+    pos, table, win, grad = to_gpu(p["pos"]), to_gpu(p["table"]), to_gpu(p["window"]), to_gpu(p["grad"])
+    n, levels = pos.shape[0], table.shape[0]
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
+    wp, wb = (ws.data_ptr(), ws_bytes) if ws is not None else (None, 0)
+    tg = torch.full_like(table, float("nan"))  # the library must clear it itself
+    st = torch.cuda.current_stream().cuda_stream
+    if dpos is None:
+        rc = lib.penc_backward(d, 2, n, levels, cap, pos.data_ptr(), table.data_ptr(), fp.m_scale_factor.data_ptr(),
+                               fp.m_random_shift_per_level.data_ptr(), win.data_ptr(), grad.data_ptr(), tg.data_ptr(),
+                               None, wp, wb, st)
+    else:
+        q = to_gpu(dpos)
+        rc = lib.penc_double_backward_from_positions(d, 2, n, levels, cap, pos.data_ptr(), table.data_ptr(),
+                                                     fp.m_scale_factor.data_ptr(), fp.m_random_shift_per_level.data_ptr(),
+                                                     win.data_ptr(), q.data_ptr(), grad.data_ptr(), tg.data_ptr(), None,
+                                                     0, wp, wb, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    return tg.cpu().numpy()
+
+
+@pytest.mark.parametrize("ws_bytes", [0, 4096, 40_000, 300_000, 3_000_000, 64_000_000])
+def test_table_gradient_does_not_depend_on_the_workspace(ws_bytes):
+    """No workspace (direct atomics), one too small to use, ones that force many passes and full
+    bins (spill to atomics), and a roomy one must all give the same sums."""
+    d, cap = 3, 1 << 15
+    p = random_problem(d, 30000, 9, cap, seed=3, sigma_range=(1.0, 1e-3))
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    got = _table_grads_with_workspace(enc, p, ws_bytes, d, cap)
+    assert_sum_close(got, want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, workspace {ws_bytes}")
+    want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    got = _table_grads_with_workspace(enc, p, ws_bytes, d, cap, dpos=p["dpos"])
+    assert_sum_close(got, want["grad64"], want["abs64"], SUM_RTOL, f"double-backward table gradient, workspace {ws_bytes}")
+
+
+def test_misaligned_workspace_and_odd_capacity():
+    d, cap = 4, 50000  # not a multiple of the bin size: the last bin is partial
+    p = random_problem(d, 20000, 6, cap, seed=8, sigma_range=(1.0, 1e-3))
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, fp = make_encoding(d, p["sigmas"], p["shift"])
+    from permutohedral_encoding_amd import _native
+    lib = _native.lib()
+    pos, table, win, grad = to_gpu(p["pos"]), to_gpu(p["table"]), to_gpu(p["window"]), to_gpu(p["grad"])
+    ws = torch.empty(8_000_000 + 64, dtype=torch.uint8, device="cuda")
+    tg = torch.empty_like(table)
+    rc = lib.penc_backward(d, 2, 20000, 6, cap, pos.data_ptr(), table.data_ptr(), fp.m_scale_factor.data_ptr(),
+                           fp.m_random_shift_per_level.data_ptr(), win.data_ptr(), grad.data_ptr(), tg.data_ptr(), None,
+                           ws.data_ptr() + 13, 8_000_000, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")

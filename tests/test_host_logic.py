@@ -56,11 +56,17 @@ def test_argument_validation_without_a_gpu():
     assert lib.penc_forward(3, 2, 1 << 30, 24, 16, p, p, p, p, p, p, 0, 1.0, None) == 2
     assert lib.penc_forward(3, 2, 10, 2, 16, z, p, p, p, p, p, 0, 1.0, None) == 1
     assert lib.penc_forward(3, 2, 10, 2, 16, p, p + 4, p, p, p, p, 0, 1.0, None) == 5
-    assert lib.penc_backward(3, 2, 10, 2, 16, p, p, p, p, p, p, z, z, None) == 1
-    assert lib.penc_backward(3, 2, 10, 2, 16, p, z, p, p, p, p, z, p, None) == 1
-    assert lib.penc_double_backward_from_positions(3, 2, 10, 2, 16, p, p, p, p, p, p, p, z, z, 0, None) == 1
+    assert lib.penc_backward(3, 2, 10, 2, 16, p, p, p, p, p, p, z, z, None, 0, None) == 1
+    assert lib.penc_backward(3, 2, 10, 2, 16, p, z, p, p, p, p, z, p, None, 0, None) == 1
+    assert lib.penc_double_backward_from_positions(3, 2, 10, 2, 16, p, p, p, p, p, p, p, z, z, 0, None, 0, None) == 1
     assert lib.penc_simplex_debug(3, 0, 2, 16, p, p, p, z, z, z, z, None) == 2
     assert lib.penc_scale_factors(3, 2, z, p) == 1
+    # workspace sizing: grows with the levels per pass, 0 when the capacity cannot be binned
+    w1 = lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 1)
+    w4 = lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 4)
+    assert 0 < w1 < w4 <= 4 * w1 and lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 100) <= 24 * w1
+    assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 22, 4) == 0
+    assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 0) == w4
 
 
 @pytest.mark.parametrize("d", range(2, 9))
