@@ -26,7 +26,7 @@
 
 namespace penc {
 
-constexpr int kDefaultLevelsPerPass = 4;  // levels binned per pass when the caller lets the library size the workspace
+constexpr int kDefaultLevelsPerPass = 1 << 20;  // by default the suggested workspace bins all levels in one pass (measured fastest)
 
 __device__ __forceinline__ float2 load_vertex(const float* __restrict__ level_table, uint32_t slot) {
     return *reinterpret_cast<const float2*>(level_table + 2 * static_cast<size_t>(slot));
@@ -359,7 +359,7 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, void*
 
 inline int reduce_bins(const BinPlan& p, const float* window, int first_level, int n_levels_in_pass, int capacity,
                        float* table_grad, hipStream_t st) {
-    hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass, kReduceSplit), dim3(kReduceBlock), 0, st,
+    hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass), dim3(kReduceBlock), 0, st,
                        p.target, window, static_cast<uint32_t>(capacity), table_grad, first_level);
     return check_launch();
 }

@@ -38,8 +38,7 @@ constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
 constexpr int kBinSlotsLog2 = 12;      // slots per bin: 4096 (32 KiB of sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
 constexpr int kMaxBins = 256;          // bins per level; capacities above kMaxBins*kBinSlots are not binned
-constexpr int kReduceBlock = 512;      // threads of a bin_reduce_kernel workgroup
-constexpr int kReduceSplit = 4;        // workgroups that share one bin in bin_reduce_kernel
+constexpr int kReduceBlock = 1024;     // threads of a bin_reduce_kernel workgroup
 
 struct BinRecord {
     uint32_t slot_in_bin;
@@ -118,7 +117,32 @@ __device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad,
     }
 }
 
-// LDS state of a scattering workgroup.
+// Two fp32 sums packed in 64 bits, updated with a compare-and-swap loop: ds_cmpst_rtn_b64 runs at
+// integer-atomic speed, where two ds_add_f32 would cost about 6 clocks per lane.  Only for cells
+// that few lanes hit at the same time.
+typedef unsigned long long packed_pair;
+
+__device__ __forceinline__ packed_pair pack_pair(float a0, float a1) {
+    return static_cast<packed_pair>(__builtin_bit_cast(uint32_t, a0)) |
+           (static_cast<packed_pair>(__builtin_bit_cast(uint32_t, a1)) << 32);
+}
+__device__ __forceinline__ float pair_lo(packed_pair v) { return __builtin_bit_cast(float, static_cast<uint32_t>(v)); }
+__device__ __forceinline__ float pair_hi(packed_pair v) { return __builtin_bit_cast(float, static_cast<uint32_t>(v >> 32)); }
+
+__device__ __forceinline__ void lds_pair_add(packed_pair* cell, float a0, float a1) {
+    packed_pair seen = *cell;
+    for (;;) {
+        const packed_pair want = pack_pair(pair_lo(seen) + a0, pair_hi(seen) + a1);
+        const packed_pair got = atomicCAS(cell, seen, want);
+        if (got == seen) break;
+        seen = got;
+    }
+}
+
+// LDS state of a scattering workgroup.  The accumulate cache adds with ds_add_f32 although that
+// instruction is slow: its lines are hit by many lanes at once (that is what the cache is for), and
+// a compare-and-swap loop degrades quadratically under such contention (measured: 10-40x slower
+// on the coarsest levels).  The bins of stage 2, whose slots are spread out, use the CAS loop.
 struct ScatterState {
     int tag[kCacheLines];
     float val[kCacheLines][2];
@@ -214,14 +238,16 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
     }
 }
 
-// Second kernel of stage 2: kReduceSplit workgroups per (bin, level) sum the bin's records in LDS
-// and add the bin's slot range into the gradient.  Sums are kept as two floats packed in 64 bits
-// and updated with a compare-and-swap loop (ds_cmpst_rtn_b64), which runs at integer-atomic speed.
-// Each wavefront takes whole segments (one per scattering workgroup), so its loads are contiguous.
+// Second kernel of stage 2: one workgroup per (bin, level) sums the bin's records in LDS and adds
+// the bin's slot range into the gradient.  Each wavefront takes whole segments (one per scattering
+// workgroup), so its loads are contiguous; a segment's records are fetched four wave-widths at a
+// time so that several loads are in flight.  Nothing else touches the gradient while this kernel
+// runs (the scattering kernel before it has completed, and bins do not overlap), so the final add
+// is a plain coalesced read-modify-write.
 __global__ void __launch_bounds__(kReduceBlock)
 bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity,
                   float* __restrict__ table_grad, int first_level) {
-    __shared__ unsigned long long acc[kBinSlots];
+    __shared__ packed_pair acc[kBinSlots];
     const uint32_t bin = blockIdx.x;
     const int level = first_level + blockIdx.y;
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
@@ -229,36 +255,35 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) acc[s] = 0ull;
     __syncthreads();
     constexpr uint32_t kWaves = kReduceBlock / 64;
+    constexpr uint32_t kUnroll = 4;
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
     const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
-    for (uint32_t g = blockIdx.z * kWaves + wave; g < bins.n_groups; g += kWaves * kReduceSplit) {
+    for (uint32_t g = wave; g < bins.n_groups; g += kWaves) {
         const uint32_t count = counts[g];
         const BinRecord* seg = recs + static_cast<size_t>(g) * bins.segment_capacity;
-        for (uint32_t i = lane; i < count; i += 64) {
-            const BinRecord rec = seg[i];
-            unsigned long long* cell = &acc[rec.slot_in_bin];
-            unsigned long long seen = *cell;
-            for (;;) {
-                const float s0 = __builtin_bit_cast(float, static_cast<uint32_t>(seen)) + rec.a0;
-                const float s1 = __builtin_bit_cast(float, static_cast<uint32_t>(seen >> 32)) + rec.a1;
-                const unsigned long long want = static_cast<unsigned long long>(__builtin_bit_cast(uint32_t, s0)) |
-                                                (static_cast<unsigned long long>(__builtin_bit_cast(uint32_t, s1)) << 32);
-                const unsigned long long got = atomicCAS(cell, seen, want);
-                if (got == seen) break;
-                seen = got;
+        for (uint32_t base = 0; base < count; base += 64 * kUnroll) {
+            BinRecord rec[kUnroll];
+#pragma unroll
+            for (uint32_t u = 0; u < kUnroll; ++u) {
+                const uint32_t i = base + u * 64 + lane;
+                rec[u] = seg[i < count ? i : 0];
             }
+#pragma unroll
+            for (uint32_t u = 0; u < kUnroll; ++u)
+                if (base + u * 64 + lane < count) lds_pair_add(&acc[rec[u].slot_in_bin], rec[u].a0, rec[u].a1);
         }
     }
     __syncthreads();
-    float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
+    float2* level_grad = reinterpret_cast<float2*>(table_grad + static_cast<size_t>(level) * capacity * 2);
     const uint32_t slot0 = bin << kBinSlotsLog2;
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
-        const unsigned long long v = acc[s];
+        const packed_pair v = acc[s];
         if (v != 0ull && slot0 + s < capacity) {
-            float* g = level_grad + 2 * static_cast<size_t>(slot0 + s);
-            global_add(g, __builtin_bit_cast(float, static_cast<uint32_t>(v)));
-            global_add(g + 1, __builtin_bit_cast(float, static_cast<uint32_t>(v >> 32)));
+            float2 g = level_grad[slot0 + s];
+            g.x += pair_lo(v);
+            g.y += pair_hi(v);
+            level_grad[slot0 + s] = g;
         }
     }
 }
