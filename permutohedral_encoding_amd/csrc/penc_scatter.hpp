@@ -5,8 +5,10 @@
 //     whatever the number of lanes in the segment (1..16), the scope or the footprint; the chip
 //     retires about 21 G such requests/s.  A level with many distinct slots is therefore bound
 //     by requests, not bytes.
-//   * ds_add_f32 retires about one lane every 3 clocks per CU, 30 times slower than integer LDS
-//     atomics (ds_add_u32, ds_cmpst_b32/b64) and than plain LDS reads and writes.
+//   * ds_add_f32 retires about one lane every 3 clocks per CU, whatever the addresses: 30 times
+//     slower than integer LDS atomics (ds_add_u32, ds_cmpst_b32/b64) and plain LDS accesses, and
+//     5-20 times slower than ds_add_f64 (1.5 lanes/clock when 8 addresses take all the traffic,
+//     3 for random addresses, 7.5 without bank conflicts).
 //
 // Hence three stages, each taking what the previous one could not combine:
 //   1. Accumulate cache in LDS.  Every workgroup keeps a small open-addressed table
@@ -139,21 +141,22 @@ __device__ __forceinline__ void lds_pair_add(packed_pair* cell, float a0, float 
     }
 }
 
-// LDS state of a scattering workgroup.  The accumulate cache adds with ds_add_f32 although that
-// instruction is slow: its lines are hit by many lanes at once (that is what the cache is for), and
-// a compare-and-swap loop degrades quadratically under such contention (measured: 10-40x slower
-// on the coarsest levels).  The bins of stage 2, whose slots are spread out, use the CAS loop.
+// LDS state of a scattering workgroup.  The accumulate cache sums in fp64 with ds_add_f64: its
+// lines are hit by many lanes at once (that is what the cache is for), where a compare-and-swap
+// loop degrades quadratically (measured: 10-40x slower on the coarsest levels) and ds_add_f32 is
+// slow on this chip.  The fp64 partial sums are rounded to fp32 once, when the cache is flushed.
+// The bins of stage 2, whose slots are spread out, use the CAS loop.
 struct ScatterState {
     int tag[kCacheLines];
-    float val[kCacheLines][2];
+    double val[kCacheLines][2];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
 };
 
 __device__ __forceinline__ void scatter_begin(ScatterState& c) {
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         c.tag[e] = -1;
-        c.val[e][0] = 0.0f;
-        c.val[e][1] = 0.0f;
+        c.val[e][0] = 0.0;
+        c.val[e][1] = 0.0;
     }
     for (int b = threadIdx.x; b < kMaxBins; b += kScatterBlock) c.bin_count[b] = 0u;
     __syncthreads();
@@ -201,8 +204,8 @@ __device__ __forceinline__ void scatter_tile(ScatterState& c, float* __restrict_
                 if (owner == -1) owner = static_cast<int>(slot[r]);
             }
             if (owner == static_cast<int>(slot[r])) {
-                __hip_atomic_fetch_add(&c.val[e][0], x0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_fetch_add(&c.val[e][1], x1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&c.val[e][0], static_cast<double>(x0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&c.val[e][1], static_cast<double>(x1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             } else {
                 miss = true;
             }
@@ -221,7 +224,7 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         const int owner = c.tag[e];
         if (owner != -1) {
-            const float v0 = c.val[e][0], v1 = c.val[e][1];
+            const float v0 = static_cast<float>(c.val[e][0]), v1 = static_cast<float>(c.val[e][1]);
             const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
             if (!binned) {
                 float* g = level_grad + 2 * static_cast<size_t>(owner);
