@@ -37,7 +37,7 @@ constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wa
 constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
 constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
 constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
-constexpr int kBinSlotsLog2 = 12;      // slots per bin: 4096 (32 KiB of sums in LDS)
+constexpr int kBinSlotsLog2 = 14;      // slots per bin: 16384 (128 KiB of sums in LDS): fewer, longer record runs per wave
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
 constexpr int kMaxBins = 256;          // bins per level; capacities above kMaxBins*kBinSlots are not binned
 constexpr int kReduceBlock = 1024;     // threads of a bin_reduce_kernel workgroup
