@@ -18,7 +18,7 @@
 //      cache is appended, as a 12-byte record, to the bin of its slot range (each workgroup has a
 //      private segment in every bin, so appending costs one LDS counter increment and one
 //      store); a second kernel (bin_reduce_kernel) reads each bin back coalesced, sums it in
-//      LDS, and adds the range into the gradient with dense atomics (8 slots per request).  This
+//      LDS (fp64), and adds the range into the gradient with coalesced read-modify-writes.  This
 //      turns the random scatter of the fine levels into streaming traffic.
 //   3. Direct global atomics, with the two features of a slot in one instruction (lane pairs),
 //      for whatever is left: no workspace, capacity too large for binning, or a full bin.
@@ -37,9 +37,9 @@ constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wa
 constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
 constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
 constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
-constexpr int kBinSlotsLog2 = 14;      // slots per bin: 16384 (128 KiB of sums in LDS): fewer, longer record runs per wave
+constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
-constexpr int kMaxBins = 256;          // bins per level; capacities above kMaxBins*kBinSlots are not binned
+constexpr int kMaxBins = 512;          // bins per level; capacities above kMaxBins*kBinSlots (2^22) are not binned
 constexpr int kReduceBlock = 1024;     // threads of a bin_reduce_kernel workgroup
 
 struct BinRecord {
@@ -119,33 +119,10 @@ __device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad,
     }
 }
 
-// Two fp32 sums packed in 64 bits, updated with a compare-and-swap loop: ds_cmpst_rtn_b64 runs at
-// integer-atomic speed, where two ds_add_f32 would cost about 6 clocks per lane.  Only for cells
-// that few lanes hit at the same time.
-typedef unsigned long long packed_pair;
-
-__device__ __forceinline__ packed_pair pack_pair(float a0, float a1) {
-    return static_cast<packed_pair>(__builtin_bit_cast(uint32_t, a0)) |
-           (static_cast<packed_pair>(__builtin_bit_cast(uint32_t, a1)) << 32);
-}
-__device__ __forceinline__ float pair_lo(packed_pair v) { return __builtin_bit_cast(float, static_cast<uint32_t>(v)); }
-__device__ __forceinline__ float pair_hi(packed_pair v) { return __builtin_bit_cast(float, static_cast<uint32_t>(v >> 32)); }
-
-__device__ __forceinline__ void lds_pair_add(packed_pair* cell, float a0, float a1) {
-    packed_pair seen = *cell;
-    for (;;) {
-        const packed_pair want = pack_pair(pair_lo(seen) + a0, pair_hi(seen) + a1);
-        const packed_pair got = atomicCAS(cell, seen, want);
-        if (got == seen) break;
-        seen = got;
-    }
-}
-
 // LDS state of a scattering workgroup.  The accumulate cache sums in fp64 with ds_add_f64: its
 // lines are hit by many lanes at once (that is what the cache is for), where a compare-and-swap
 // loop degrades quadratically (measured: 10-40x slower on the coarsest levels) and ds_add_f32 is
 // slow on this chip.  The fp64 partial sums are rounded to fp32 once, when the cache is flushed.
-// The bins of stage 2, whose slots are spread out, use the CAS loop.
 struct ScatterState {
     int tag[kCacheLines];
     double val[kCacheLines][2];
@@ -241,21 +218,25 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
     }
 }
 
-// Second kernel of stage 2: one workgroup per (bin, level) sums the bin's records in LDS and adds
-// the bin's slot range into the gradient.  Each wavefront takes whole segments (one per scattering
-// workgroup), so its loads are contiguous; a segment's records are fetched four wave-widths at a
-// time so that several loads are in flight.  Nothing else touches the gradient while this kernel
-// runs (the scattering kernel before it has completed, and bins do not overlap), so the final add
-// is a plain coalesced read-modify-write.
+// Second kernel of stage 2: one workgroup per (bin, level) sums the bin's records in LDS (fp64,
+// ds_add_f64: a few hot slots must not serialise the whole bin, which rules out a compare-and-swap
+// loop) and adds the bin's slot range into the gradient.  Each wavefront takes whole segments (one
+// per scattering workgroup), so its loads are contiguous; a segment's records are fetched four
+// wave-widths at a time so that several loads are in flight.  Nothing else touches the gradient
+// while this kernel runs (the scattering kernel before it has completed, and bins do not
+// overlap), so the final add is a plain coalesced read-modify-write.
 __global__ void __launch_bounds__(kReduceBlock)
 bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity,
                   float* __restrict__ table_grad, int first_level) {
-    __shared__ packed_pair acc[kBinSlots];
+    __shared__ double acc[kBinSlots][2];
     const uint32_t bin = blockIdx.x;
     const int level = first_level + blockIdx.y;
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
     const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
-    for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) acc[s] = 0ull;
+    for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
+        acc[s][0] = 0.0;
+        acc[s][1] = 0.0;
+    }
     __syncthreads();
     constexpr uint32_t kWaves = kReduceBlock / 64;
     constexpr uint32_t kUnroll = 4;
@@ -274,18 +255,22 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
             }
 #pragma unroll
             for (uint32_t u = 0; u < kUnroll; ++u)
-                if (base + u * 64 + lane < count) lds_pair_add(&acc[rec[u].slot_in_bin], rec[u].a0, rec[u].a1);
+                if (base + u * 64 + lane < count) {
+                    double* cell = acc[rec[u].slot_in_bin];
+                    __hip_atomic_fetch_add(cell, static_cast<double>(rec[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(cell + 1, static_cast<double>(rec[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
         }
     }
     __syncthreads();
     float2* level_grad = reinterpret_cast<float2*>(table_grad + static_cast<size_t>(level) * capacity * 2);
     const uint32_t slot0 = bin << kBinSlotsLog2;
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
-        const packed_pair v = acc[s];
-        if (v != 0ull && slot0 + s < capacity) {
+        const double v0 = acc[s][0], v1 = acc[s][1];
+        if ((v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity) {
             float2 g = level_grad[slot0 + s];
-            g.x += pair_lo(v);
-            g.y += pair_hi(v);
+            g.x += static_cast<float>(v0);
+            g.y += static_cast<float>(v1);
             level_grad[slot0 + s] = g;
         }
     }
