@@ -61,6 +61,12 @@ __device__ __forceinline__ Vertices<D> load_vertices(const float* __restrict__ l
 
 // ------------------------------------------------------------------------------------------
 // forward (EncodingGPU.cuh:68-256)
+//
+// Measured alternatives to one thread per (point, level), all slower or equal: 2 or 4 points per
+// thread (more loads in flight per lane: no gain, the kernel already runs at the rate this GPU
+// sustains for random 8-byte loads from a 2 MiB slice); walking the levels inside the thread with
+// the positions kept in registers (20% slower at 2^20 points, 3x slower at 2^16: fewer, longer
+// waves lose more than the re-read positions cost).
 
 template <int D>
 __global__ void __launch_bounds__(kBlock)
@@ -134,7 +140,9 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
             PENC_INDEX(r);
             slot[r] = to_slot(h[r], capacity, cap_mask);
         });
-        scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
+        const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t), slot,
+                                              w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
+        if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
     }
     scatter_end(state, level_grad, bins, blockIdx.x);
 }
@@ -224,7 +232,9 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
             }
             if constexpr (kTableGrad) {
                 const float g0 = g0p[nn], g1 = g1p[nn];
-                scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, slot, wr * g0, wr * g1);
+                const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t),
+                                                      slot, wr * g0, wr * g1);
+                if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
             }
         }
         if (kGradGrad && active) {
@@ -357,6 +367,8 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, void*
     return p;
 }
 
+// Running consecutive passes on two streams (scatter pass p+1 while pass p is reduced) was tried and
+// measured 10-15% slower than one pass over all levels on one stream; hence a single stream.
 inline int reduce_bins(const BinPlan& p, const float* window, int first_level, int n_levels_in_pass, int capacity,
                        float* table_grad, hipStream_t st) {
     hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass), dim3(kReduceBlock), 0, st,

@@ -127,6 +127,7 @@ struct ScatterState {
     int tag[kCacheLines];
     double val[kCacheLines][2];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
+    uint32_t hits;                 // contributions the cache has absorbed into existing lines
 };
 
 __device__ __forceinline__ void scatter_begin(ScatterState& c) {
@@ -136,6 +137,7 @@ __device__ __forceinline__ void scatter_begin(ScatterState& c) {
         c.val[e][1] = 0.0;
     }
     for (int b = threadIdx.x; b < kMaxBins; b += kScatterBlock) c.bin_count[b] = 0u;
+    if (threadIdx.x == 0) c.hits = 0u;
     __syncthreads();
 }
 
@@ -154,43 +156,78 @@ __device__ __forceinline__ bool append_record(ScatterState& c, const BinTarget& 
     return true;
 }
 
+// Looks `slot` up in the accumulate cache, claiming a free line if there is one.  Two candidate
+// lines per slot (two-choice hashing): with one, a level with a few hundred distinct slots already
+// loses several of them to collisions, and those are exactly the slots every wave keeps hitting.
+// Returns the line, or -1 when both candidates belong to other slots; `found` tells whether the
+// line already held the slot (a hit, as opposed to a claim).
+__device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& found) {
+    const int want = static_cast<int>(slot);
+    int e = static_cast<int>(slot & (kCacheLines - 1));
+    found = false;
+#pragma unroll
+    for (int probe = 0; probe < 2; ++probe) {
+        int owner = c.tag[e];
+        if (owner == want) {
+            found = true;
+            return e;
+        }
+        if (owner == -1) {
+            owner = atomicCAS(&c.tag[e], -1, want);
+            if (owner == -1 || owner == want) return e;
+        }
+        e = static_cast<int>((slot * 0x9E3779B1u) >> (32 - 11)) & (kCacheLines - 1);
+    }
+    return -1;
+}
+static_assert(kCacheLines == 1 << 11, "cache_find derives its second line from the top 11 bits of a product");
+
 // One tile's D+1 contributions per thread through stages 1-3.  All 64 lanes of every wave must
 // call it together; `active` is false for lanes that carry no point (tail of the last tile), which
-// only take part in the wave-wide steps.
+// only take part in the wave-wide steps.  `use_cache` (wave-uniform) is false once the workgroup
+// has seen that the cache does not hit at this level; the return value is the number of hits of
+// this wave in this tile.
 template <int D>
-__device__ __forceinline__ void scatter_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
-                                             uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
-                                             fvec<D + 1> a1) {
+__device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+                                                 uint32_t group, bool active, bool use_cache, uvec<D + 1> slot,
+                                                 fvec<D + 1> a0, fvec<D + 1> a1) {
+    uint32_t hits = 0;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
-        // stage 1; a wave whose lanes all hit one slot reduces with DPP and lets lane 63 add the sum
-        const uint32_t first = __builtin_amdgcn_readfirstlane(slot[r]);
         float x0 = a0[r], x1 = a1[r];
-        bool act = active;
-        if (__all(active && slot[r] == first)) {
-            x0 = wave_sum_to_last_lane(x0);
-            x1 = wave_sum_to_last_lane(x1);
-            act = (threadIdx.x & 63) == 63;
-        }
-        bool miss = false;
-        if (act) {
-            const int e = static_cast<int>(slot[r] & (kCacheLines - 1));
-            int owner = c.tag[e];
-            if (owner == -1) {
-                owner = atomicCAS(&c.tag[e], -1, static_cast<int>(slot[r]));
-                if (owner == -1) owner = static_cast<int>(slot[r]);
+        bool miss = active;
+        if (use_cache) {
+            // stage 1; a wave whose lanes all hit one slot reduces with DPP and lets lane 63 add the sum
+            const uint32_t first = __builtin_amdgcn_readfirstlane(slot[r]);
+            if (__all(active && slot[r] == first)) {
+                x0 = wave_sum_to_last_lane(x0);
+                x1 = wave_sum_to_last_lane(x1);
+                miss = (threadIdx.x & 63) == 63;
+                hits += 63;  // the other lanes were absorbed without touching the cache
             }
-            if (owner == static_cast<int>(slot[r])) {
-                __hip_atomic_fetch_add(&c.val[e][0], static_cast<double>(x0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_fetch_add(&c.val[e][1], static_cast<double>(x1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            } else {
-                miss = true;
+            bool found = false;
+            if (miss) {
+                const int e = cache_find(c, slot[r], found);
+                if (e >= 0) {
+                    __hip_atomic_fetch_add(&c.val[e][0], static_cast<double>(x0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&c.val[e][1], static_cast<double>(x1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    miss = false;
+                }
             }
+            hits += __popcll(__ballot(found));
         }
         // stage 2, then stage 3 for what stage 2 could not take
         if (miss && bins.records != nullptr) miss = !append_record(c, bins, group, slot[r], x0, x1);
         if (__any(miss)) global_add_pairs(level_grad, miss, slot[r], x0, x1);
     });
+    return hits;
+}
+
+// The workgroup-wide decision whether stage 1 is worth its LDS traffic at this level: after the
+// first tile, keep using the cache only while at least one contribution in eight hits.
+template <int D>
+__device__ __forceinline__ bool cache_pays(const ScatterState& c, int tiles_done) {
+    return tiles_done == 0 || c.hits * 8u >= static_cast<uint32_t>(tiles_done) * kScatterBlock * (D + 1);
 }
 
 // After the last tile: flushes the accumulate cache (through the bins when there are any) and
@@ -243,23 +280,29 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
     const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
-    for (uint32_t g = wave; g < bins.n_groups; g += kWaves) {
-        const uint32_t count = counts[g];
-        const BinRecord* seg = recs + static_cast<size_t>(g) * bins.segment_capacity;
-        for (uint32_t base = 0; base < count; base += 64 * kUnroll) {
-            BinRecord rec[kUnroll];
+    // segments g = wave, wave + kWaves, ...; their record counts are fetched 64 at a time (one per
+    // lane) so that no segment has to wait for its own count
+    for (uint32_t g0 = wave; g0 < bins.n_groups; g0 += kWaves * 64) {
+        const uint32_t mine = g0 + lane * kWaves;
+        const uint32_t my_count = mine < bins.n_groups ? counts[mine] : 0u;
+        for (uint32_t k = 0; k < 64 && g0 + k * kWaves < bins.n_groups; ++k) {
+            const uint32_t count = __builtin_amdgcn_readlane(my_count, k);
+            const BinRecord* seg = recs + static_cast<size_t>(g0 + k * kWaves) * bins.segment_capacity;
+            for (uint32_t base = 0; base < count; base += 64 * kUnroll) {
+                BinRecord rec[kUnroll];
 #pragma unroll
-            for (uint32_t u = 0; u < kUnroll; ++u) {
-                const uint32_t i = base + u * 64 + lane;
-                rec[u] = seg[i < count ? i : 0];
-            }
-#pragma unroll
-            for (uint32_t u = 0; u < kUnroll; ++u)
-                if (base + u * 64 + lane < count) {
-                    double* cell = acc[rec[u].slot_in_bin];
-                    __hip_atomic_fetch_add(cell, static_cast<double>(rec[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(cell + 1, static_cast<double>(rec[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                for (uint32_t u = 0; u < kUnroll; ++u) {
+                    const uint32_t i = base + u * 64 + lane;
+                    rec[u] = seg[i < count ? i : 0];
                 }
+#pragma unroll
+                for (uint32_t u = 0; u < kUnroll; ++u)
+                    if (base + u * 64 + lane < count) {
+                        double* cell = acc[rec[u].slot_in_bin];
+                        __hip_atomic_fetch_add(cell, static_cast<double>(rec[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        __hip_atomic_fetch_add(cell + 1, static_cast<double>(rec[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+            }
         }
     }
     __syncthreads();
