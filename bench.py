@@ -158,7 +158,10 @@ def main():
                               P(win), P(out), 0, 1.0, stream)
         assert rc == 0, rc
 
-    ws_bytes = int(lib.penc_scatter_workspace_bytes(d, n, levels, cap, args.levels_per_pass)) if args.levels_per_pass >= 0 else 0
+    ws_bytes = 0
+    if args.levels_per_pass >= 0:
+        ws_bytes = max(int(lib.penc_scatter_workspace_bytes(d, n, levels, cap, args.levels_per_pass)),
+                       int(lib.penc_positions_workspace_bytes(d, n, levels)))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
 
     def backward():

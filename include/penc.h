@@ -69,6 +69,13 @@ int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* s
 size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
                                     int levels_per_pass);
 
+/* Size of `workspace` that lets penc_backward compute positions_grad in groups of a few levels
+ * (partial sums in the workspace, then one deterministic reduction) instead of one thread walking
+ * all levels; 0 when there is nothing to gain.  A workspace serving both gradients needs the larger
+ * of the two sizes.  No counterpart in the reference (it sums levels with atomics,
+ * EncodingGPU.cuh:745-750). */
+size_t penc_positions_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels);
+
 /* Slice: sliced_values[l][f][n] = sum over the D+1 simplex vertices of
  * lattice_values[l][slot][f] * barycentric * anneal_window[l]; extra levels copy
  * positions * points_scaling (zero-padded).

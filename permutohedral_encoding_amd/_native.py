@@ -27,6 +27,7 @@ _SIGNATURES = {
                                     ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
     "penc_scatter_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                                        ctypes.c_int]),
+    "penc_positions_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int]),
     "penc_backward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                      _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                      ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
@@ -85,11 +86,16 @@ def scale_factors(pos_dim, sigmas):
 LEVELS_PER_PASS = 0
 
 
-def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device):
+def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device, table_grad=True, positions_grad=False):
+    """Scratch memory for one gradient call (None when the library would not use any)."""
     if LEVELS_PER_PASS < 0:
         return None
-    nbytes = int(lib().penc_scatter_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels), int(capacity),
-                                                    int(LEVELS_PER_PASS)))
+    nbytes = 0
+    if table_grad:
+        nbytes = int(lib().penc_scatter_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels), int(capacity),
+                                                        int(LEVELS_PER_PASS)))
+    if positions_grad:
+        nbytes = max(nbytes, int(lib().penc_positions_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels))))
     if nbytes == 0:
         return None
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -223,7 +229,7 @@ class EncodingWrapper:
         if lv_grad is None and pos_grad is None:
             return None, None
         with torch.cuda.device(pos.device):
-            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device) if lv_grad is not None else None
+            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None)
             _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
                                        _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
                                        _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(pos_grad),

@@ -26,6 +26,11 @@
 
 namespace penc {
 
+#ifndef PENC_POS_LEVELS_PER_GROUP
+#define PENC_POS_LEVELS_PER_GROUP 2
+#endif
+constexpr int kPosLevelsPerGroup = PENC_POS_LEVELS_PER_GROUP;  // levels one position-gradient thread sums
+
 constexpr int kDefaultLevelsPerPass = 1 << 20;  // by default the suggested workspace bins all levels in one pass (measured fastest)
 
 __device__ __forceinline__ float2 load_vertex(const float* __restrict__ level_table, uint32_t slot) {
@@ -150,18 +155,26 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
 // ------------------------------------------------------------------------------------------
 // backward w.r.t. positions (EncodingGPU.cuh:530-769)
 
+// One thread per (point, group of consecutive levels): the levels of the group are summed in
+// registers and stored once, at out[group][point][D].  With a single group (no workspace) `out` is
+// the position gradient itself; otherwise it is a partial buffer that reduce_level_groups_kernel
+// sums, in ascending group order, so the result is deterministic either way.  Small groups keep
+// the whole chip on the same few levels at a time (their table slices stay in L2) and give the
+// launch many more, shorter waves than one thread per point walking all levels.
 template <int D>
 __global__ void __launch_bounds__(kBlock)
-backward_pos_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
+backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t capacity, uint32_t cap_mask,
                     const float* __restrict__ positions, const float* __restrict__ table,
                     const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                     const float* __restrict__ window, const float* __restrict__ grad_sliced,
-                    float* __restrict__ positions_grad) {
+                    float* __restrict__ out) {
     const int n = blockIdx.x * kBlock + threadIdx.x;
     if (n >= n_points) return;
     const fvec<D> pos = load_point<D>(positions, n);
     fvec<D> total = 0.0f;
-    for (int level = 0; level < n_levels; ++level) {
+    const int first = blockIdx.y * levels_per_group;
+    const int last = first + levels_per_group < n_levels ? first + levels_per_group : n_levels;
+    for (int level = first; level < last; ++level) {
         const float w_level = window[level];
         if (w_level == 0.0f) continue;
         const float* sf = scale_factor + level * D;
@@ -173,9 +186,21 @@ backward_pos_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_
         const fvec<D + 1> dB = (v.f0 * w_level) * g0 + (v.f1 * w_level) * g1;  // :688-689
         total += bary_grad_to_pos_grad<D>(s.rank, dB, sf);
     }
-    float* o = positions_grad + static_cast<size_t>(n) * D;
+    float* o = out + (static_cast<size_t>(blockIdx.y) * n_points + n) * D;
     static_for<D>(PENC_BODY(i) {
-        PENC_INDEX(i); o[i] = total[i]; });
+        PENC_INDEX(i);
+        o[i] = total[i];
+    });
+}
+
+__global__ void __launch_bounds__(kBlock)
+reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size_t n_values, float* __restrict__ out) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n_values; i += stride) {
+        float acc = partial[i];
+        for (int g = 1; g < n_groups; ++g) acc += partial[static_cast<size_t>(g) * n_values + i];
+        out[i] = acc;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -424,6 +449,12 @@ size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_le
     return per_level * static_cast<size_t>(levels_per_pass) + 1024;
 }
 
+size_t penc_positions_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels) {
+    if (pos_dim < 2 || pos_dim > 8 || nr_positions <= 0 || nr_levels <= kPosLevelsPerGroup) return 0;
+    const size_t groups = static_cast<size_t>((nr_levels + kPosLevelsPerGroup - 1) / kPosLevelsPerGroup);
+    return groups * static_cast<size_t>(nr_positions) * pos_dim * sizeof(float) + 256;
+}
+
 int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* scale_factor_out) {
     if (!sigmas || !scale_factor_out) return PENC_ERR_NULL_POINTER;
     if (pos_dim < 1 || nr_levels < 1) return PENC_ERR_BAD_SIZE;
@@ -485,11 +516,30 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
         }
     }
     if (positions_grad) {
-        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions)), dim3(kBlock), 0,
-                                                    st, n, nr_levels, cap, mask, positions, lattice_values,
-                                                    scale_factor, random_shift, anneal_window, grad_sliced_values,
-                                                    positions_grad));
+        // levels in groups of kPosLevelsPerGroup when the workspace can hold the partial sums
+        // (the table-gradient scatter above is done with it: same stream), else one group
+        const size_t n_values = static_cast<size_t>(nr_positions) * pos_dim;
+        int per_group = nr_levels, groups = 1;
+        float* partial = positions_grad;
+        const uintptr_t ws = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
+        const int want_groups = (nr_levels + kPosLevelsPerGroup - 1) / kPosLevelsPerGroup;
+        if (workspace != nullptr && want_groups > 1 &&
+            workspace_bytes >= (ws - reinterpret_cast<uintptr_t>(workspace)) + want_groups * n_values * sizeof(float)) {
+            per_group = kPosLevelsPerGroup;
+            groups = want_groups;
+            partial = reinterpret_cast<float*>(ws);
+        }
+        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions), groups),
+                                                    dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
+                                                    lattice_values, scale_factor, random_shift, anneal_window,
+                                                    grad_sliced_values, partial));
         if (int rc = check_launch()) return rc;
+        if (groups > 1) {
+            const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
+            hipLaunchKernelGGL(reduce_level_groups_kernel, dim3(static_cast<unsigned>(want < 8192 ? want : 8192)), dim3(kBlock),
+                               0, st, partial, groups, n_values, positions_grad);
+            if (int rc = check_launch()) return rc;
+        }
     }
     return PENC_OK;
 }

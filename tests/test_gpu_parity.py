@@ -333,3 +333,26 @@ def test_misaligned_workspace_and_odd_capacity():
     assert rc == 0
     want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
     assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+
+
+def test_position_gradient_with_and_without_workspace():
+    """Level groups with partial sums (workspace) and one thread walking all levels (no workspace)
+    must agree with the oracle; the grouped result is deterministic."""
+    from permutohedral_encoding_amd import _native
+    d, cap = 4, 1 << 12
+    p = random_problem(d, 5000, 7, cap, seed=12, sigma_range=(1.0, 1e-3))  # 7 levels: a ragged last group
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    want = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])["grad64"]
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    results = []
+    for lpp in (0, -1, 0):
+        _native.LEVELS_PER_PASS = lpp
+        try:
+            _, pg = enc.backward(gpu_input(p, False, True), to_gpu(p["grad"]))
+        finally:
+            _native.LEVELS_PER_PASS = 0
+        got = pg.cpu().numpy()
+        assert np.all(np.abs(got - want) <= SUM_RTOL * (np.abs(want) + scale))
+        results.append(got)
+    assert np.array_equal(results[0], results[2])
