@@ -206,8 +206,10 @@ def main():
     phase_bytes = {"forward": ab["forward"]}
     phase_bytes["backward"] = (ab["backward_table"] if want_table else 0.0) + (ab["backward_pos"] if want_pos else 0.0)
     phase_bytes["double_backward"] = ab["double_backward"]
-    kernel_names = {"forward": "forward_kernel", "backward": "fill_zero_kernel+backward_table_kernel"
-                    if want_table and not want_pos else "backward kernels", "double_backward": "double_backward_kernel"}
+    kernel_names = {"forward": "forward_kernel",
+                    "backward": "+".join((["fill_zero_kernel", "backward_table_kernel", "bin_reduce_kernel"] if want_table else [])
+                                         + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else [])),
+                    "double_backward": "fill_zero_kernel+double_backward_kernel+bin_reduce_kernel"}
     dominant = max(phase_ms, key=phase_ms.get)
     achieved = phase_bytes[dominant] * w.point_levels / (phase_ms[dominant] * 1e-3) / 1e9
     traffic = None
@@ -243,17 +245,17 @@ def main():
     if not args.no_probes:
         result["probes"] = run_probes(torch, _native, cap, n, d + 1)
         pr = result["probes"]
-        # time the table traffic alone would take at the measured random-access rates
-        bound_s = 0.0
-        for name, _ in phases:
-            if name == "forward":
-                bound_s += w.point_levels * (d + 1) / (pr["gather_Gacc_per_s"] * 1e9)
-            elif name == "backward" and want_table:
-                bound_s += w.point_levels * 2 * (d + 1) / (pr["scatter_Gatomic_per_s"] * 1e9)
-        stream_bytes = w.point_levels * (8 + (8 if want_table else 0)) + n * d * 4 * 2 + (8.0 * cap * levels if want_table else 0)
-        bound_s += stream_bytes / (pr["copy_GBps"] * 1e9)
+        # What the table traffic alone would take if every one of the N*L*(D+1) slot accesses of each
+        # table-touching phase (gather or scatter alike) ran at the measured random 8-byte gather rate,
+        # plus the streaming traffic at the measured copy rate.
+        table_phases = sum(1 for name, _ in phases if name == "forward" or (name == "backward" and (want_table or want_pos))
+                           or name == "double_backward") + (1 if ("backward", backward) in phases and want_table and want_pos else 0)
+        bound_s = table_phases * w.point_levels * (d + 1) / (pr["gather_Gacc_per_s"] * 1e9)
+        stream_bytes = sum(phase_bytes[name] - 8 * (d + 1) * (2 if name == "double_backward" else 1) for name, _ in phases) * w.point_levels
+        bound_s += max(stream_bytes, 0.0) / (pr["copy_GBps"] * 1e9)
         result["measured_roofline"] = {"bound_ms": bound_s * 1e3, "frac": bound_s * 1e3 / ms_per_step,
-                                       "note": "random gathers/atomics at the probe rates + streaming at the copy rate"}
+                                       "note": "every table slot access at the probe's random-gather rate + streaming at "
+                                               "the probe's copy rate; frac = bound / measured step"}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w, inputs, args.cpu_sample)
     print(json.dumps(result))

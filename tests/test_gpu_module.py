@@ -112,3 +112,35 @@ def test_concat_points_module():
     assert torch.all(out[:, 15] == 0)
     out.sum().backward()  # gradient does not flow to positions through the copied columns (as in the reference)
     assert m.lattice_values.grad is not None
+
+
+def test_toy_sdf_training_with_eikonal_term():
+    """End to end through autograd, like the reference's toy example plus an eikonal term:
+    encoding -> small MLP -> SDF of a sphere; the loss uses the SDF value (first backward into the
+    table), its gradient w.r.t. positions (position backward) and the norm of that gradient (double
+    backward), with a coarse-to-fine window.  The loss must go down by a large factor."""
+    import permutohedral_encoding_amd as pe
+    torch.manual_seed(0)
+    levels = 8
+    enc = pe.PermutoEncoding(3, 1 << 14, levels, 2, np.geomspace(1.0, 0.05, levels))
+    mlp = torch.nn.Sequential(torch.nn.Linear(enc.output_dims(), 32), torch.nn.Softplus(beta=20),
+                              torch.nn.Linear(32, 1)).cuda()
+    c2f = pe.Coarse2Fine(levels)
+    opt = torch.optim.Adam(list(enc.parameters()) + list(mlp.parameters()), lr=1e-2)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    losses = []
+    for it in range(150):
+        pos = torch.rand(4096, 3, device="cuda", generator=gen).requires_grad_(True)
+        target = (pos.detach() - 0.5).norm(dim=1, keepdim=True) - 0.3
+        window = c2f(pe.map_range_val(it, 0, 100, 0.3, 1.0))
+        sdf = mlp(enc(pos, window))
+        grad, = torch.autograd.grad(sdf.sum(), pos, create_graph=True)
+        loss = ((sdf - target) ** 2).mean() + 0.05 * ((grad.norm(dim=1) - 1.0) ** 2).mean()
+        opt.zero_grad(set_to_none=True)
+        loss.backward()
+        assert enc.lattice_values.grad is not None and torch.isfinite(enc.lattice_values.grad).all()
+        assert enc.random_shift_per_level.grad is None  # the shift is a parameter only to be checkpointed
+        opt.step()
+        losses.append(loss.item())
+    assert np.mean(losses[-10:]) < 0.2 * np.mean(losses[:5]), (losses[:5], losses[-10:])
