@@ -144,3 +144,39 @@ def test_toy_sdf_training_with_eikonal_term():
         opt.step()
         losses.append(loss.item())
     assert np.mean(losses[-10:]) < 0.2 * np.mean(losses[:5]), (losses[:5], losses[-10:])
+
+
+def test_forward_and_backward_replay_in_a_hip_graph():
+    """The entry points only enqueue kernels on the given stream (the gradient is cleared by a fill
+    kernel, not a memset), so a captured step must replay to the eager results, every time."""
+    from permutohedral_encoding_amd import _native
+    from helpers import random_problem, make_encoding, gpu_input
+    d, cap = 3, 1 << 14
+    p = random_problem(d, 20000, 8, cap, seed=21, sigma_range=(1.0, 1e-3))
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    grad = to_gpu(p["grad"])
+    out_eager = enc.forward(inp)
+    tg_eager, pg_eager = enc.backward(inp, grad)
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up on the capture stream, as torch asks for
+        enc.forward(inp)
+        enc.backward(inp, grad)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = enc.forward(inp)
+        tg_g, pg_g = enc.backward(inp, grad)
+    for replay in range(3):
+        out_g.zero_()
+        tg_g.fill_(float("nan"))
+        pg_g.zero_()
+        (grad * 2).sum().item()  # unrelated eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_eager), replay
+        assert torch.equal(pg_g, pg_eager), replay
+        assert torch.allclose(tg_g, tg_eager, rtol=1e-4, atol=1e-6 * tg_eager.abs().max().item()), replay
