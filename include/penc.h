@@ -111,6 +111,12 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
                                         float* grad_grad_sliced_values, int concat_points, void* workspace,
                                         size_t workspace_bytes, void* stream);
 
+/* dst[c][r] = src[r][c] for a dense row-major rows x cols matrix with cols <= 255 (2 * levels):
+ * turns the row-major upstream gradient (N, 2(L+E)) into the grad_sliced_values layout
+ * [L+E][2][N] at streaming speed.
+ * Replaces: the strided `.contiguous()` copy of src/pytorch_modules/funcs.py:47. */
+int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream);
+
 /* Introspection for parity checks: what the kernels derive from each (level, point) before they
  * touch the table.  Outputs are [L][N][D+1]; each may be NULL.
  *   rem0, rank : the remainder-0 lattice point and the residual ranks after the hyperplane wrap

@@ -35,6 +35,7 @@ _SIGNATURES = {
                                                            ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int,
                                                            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_transpose": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
                                           _c_f32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, _c_f32p,
                                           ctypes.c_void_p]),
@@ -119,6 +120,25 @@ def _check_f32_gpu(t, name, ndim):
     _require(t.is_cuda, f"{name} should be in GPU memory. Please call .cuda() on the tensor")
     _require(t.dtype == torch.float32, f"{name} should be of type float")
     _require(t.dim() == ndim, f"{name} should have {ndim} dimensions, however it has sizes {tuple(t.shape)}")
+
+
+def level_major_gradient(grad):
+    """The contiguous (L, 2, N) tensor the gradient kernels read, from whatever autograd hands over.
+
+    The usual case is a (L, 2, N) *view* of a row-major (N, 2L) gradient (what the layer after the
+    encoding produces, seen through the module's permute+reshape): that is transposed by the
+    library at streaming speed.  Anything else takes torch's generic copy (reference: funcs.py:47).
+    """
+    if grad.is_contiguous():
+        return grad
+    levels, feat, n = grad.shape
+    cols = levels * feat
+    if (grad.is_cuda and grad.dtype == torch.float32 and grad.stride() == (feat, 1, cols) and cols <= 255 and n > 0):
+        out = torch.empty((levels, feat, n), dtype=torch.float32, device=grad.device)
+        with torch.cuda.device(grad.device):
+            _check(lib().penc_transpose(grad.data_ptr(), out.data_ptr(), n, cols, _stream()), "transpose")
+        return out
+    return grad.contiguous()
 
 
 class EncodingInput:

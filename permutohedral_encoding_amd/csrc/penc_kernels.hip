@@ -296,6 +296,38 @@ simplex_debug_kernel(int n_points, uint32_t capacity, uint32_t cap_mask, const f
     });
 }
 
+// dst[c][r] = src[r][c] for a tall matrix (rows = points, cols = 2 * levels): what turns the
+// row-major upstream gradient (N, 2L) an MLP delivers into the level-major (L, 2, N) layout the
+// kernels read (the reference does this with a strided `.contiguous()` copy,
+// src/pytorch_modules/funcs.py:47).  Each workgroup moves kTransposeRows rows through LDS: the
+// read is one contiguous chunk, every write a run of 64 consecutive floats.
+constexpr int kTransposeRows = 64;  // rows per workgroup: one wavefront-wide run per written column
+
+__global__ void __launch_bounds__(kBlock)
+transpose_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t rows, int cols) {
+    extern __shared__ float tile[];  // kTransposeRows x (cols | 1)
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTransposeRows;
+    const int n_rows = rows - row0 < kTransposeRows ? static_cast<int>(rows - row0) : kTransposeRows;
+    const int stride = cols | 1;  // odd: a column read walks all banks
+    const float* chunk = src + row0 * cols;
+    const int n_values = n_rows * cols;
+    int r = threadIdx.x / cols, c = threadIdx.x % cols;
+    const int dr = kBlock / cols, dc = kBlock % cols;
+    for (int i = threadIdx.x; i < n_values; i += kBlock) {
+        tile[r * stride + c] = chunk[i];
+        r += dr;
+        c += dc;
+        if (c >= cols) {
+            c -= cols;
+            ++r;
+        }
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane < n_rows)
+        for (int col = wave; col < cols; col += kBlock / 64) dst[static_cast<int64_t>(col) * rows + row0 + lane] = tile[lane * stride + col];
+}
+
 __global__ void __launch_bounds__(kBlock) fill_zero_kernel(float2* __restrict__ p, size_t n2) {
     const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
     for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n2; i += stride)
@@ -592,6 +624,16 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
     }
 #undef PENC_LAUNCH_DB
     return PENC_OK;
+}
+
+int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream) {
+    if (!src || !dst) return PENC_ERR_NULL_POINTER;
+    if (rows <= 0 || cols <= 0 || cols > 255 || rows > ((int64_t{1} << 31) - 1) / cols) return PENC_ERR_BAD_SIZE;
+    const size_t lds = static_cast<size_t>(kTransposeRows) * (cols | 1) * sizeof(float);
+    if (lds > 64 * 1024) return PENC_ERR_BAD_SIZE;
+    const unsigned blocks = static_cast<unsigned>((rows + kTransposeRows - 1) / kTransposeRows);
+    hipLaunchKernelGGL(transpose_kernel, dim3(blocks), dim3(kBlock), lds, static_cast<hipStream_t>(stream), src, dst, rows, cols);
+    return check_launch();
 }
 
 int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,

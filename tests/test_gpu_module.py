@@ -180,3 +180,26 @@ def test_forward_and_backward_replay_in_a_hip_graph():
         assert torch.equal(out_g, out_eager), replay
         assert torch.equal(pg_g, pg_eager), replay
         assert torch.allclose(tg_g, tg_eager, rtol=1e-4, atol=1e-6 * tg_eager.abs().max().item()), replay
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 2), (255, 48), (256, 48), (257, 48), (100000, 32), (5000, 63), (7, 1), (1000, 255)])
+def test_streaming_transpose(rows, cols):
+    from permutohedral_encoding_amd import _native
+    src = torch.randn(rows, cols, device="cuda")
+    dst = torch.empty(cols, rows, device="cuda")
+    rc = _native.lib().penc_transpose(src.data_ptr(), dst.data_ptr(), rows, cols, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert torch.equal(dst, src.t().contiguous())
+
+
+def test_level_major_gradient_paths():
+    from permutohedral_encoding_amd import _native
+    up = torch.randn(3000, 12, device="cuda")                       # row-major (N, 2L) as a linear layer delivers it
+    view = up.reshape(3000, 6, 2).permute(1, 2, 0)                   # what autograd hands to the Function
+    assert not view.is_contiguous()
+    got = _native.level_major_gradient(view)
+    assert got.is_contiguous() and torch.equal(got, view.contiguous())
+    odd = torch.randn(6, 2, 6000, device="cuda")[:, :, ::2]          # some other strided view: generic copy
+    assert torch.equal(_native.level_major_gradient(odd), odd.contiguous())
+    c = torch.randn(6, 2, 100, device="cuda")
+    assert _native.level_major_gradient(c) is c
