@@ -37,6 +37,8 @@ constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wa
 constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
 constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
 constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
+constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
+constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
 constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
 constexpr int kMaxBins = 512;          // bins per level; capacities above kMaxBins*kBinSlots (2^22) are not binned
@@ -91,6 +93,11 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v) {
     PENC_DPP_ADD(kBcast31, 0xc);
 #undef PENC_DPP_ADD
     return v;
+}
+
+// The value `v` has in lane `lane` (wave-uniform index), broadcast to all lanes.
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
 // Stage 3.  Lanes are paired (2p, 2p+1): first both lanes of a pair add the two features of the
@@ -197,13 +204,27 @@ __device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, float* __restr
         float x0 = a0[r], x1 = a1[r];
         bool miss = active;
         if (use_cache) {
-            // stage 1; a wave whose lanes all hit one slot reduces with DPP and lets lane 63 add the sum
-            const uint32_t first = __builtin_amdgcn_readfirstlane(slot[r]);
-            if (__all(active && slot[r] == first)) {
-                x0 = wave_sum_to_last_lane(x0);
-                x1 = wave_sum_to_last_lane(x1);
-                miss = (threadIdx.x & 63) == 63;
-                hits += 63;  // the other lanes were absorbed without touching the cache
+            // stage 1.  At the coarsest levels the 64 lanes of a wave hit two to six distinct slots,
+            // and LDS atomics on one address serialise (about 5 clocks per lane): so first, up to
+            // kWaveGroups times, take the slot of the first pending lane, sum the contributions of
+            // all lanes that share it with DPP, and leave the sum with that lane alone.  A group
+            // of fewer than kMinWaveGroup lanes means the wave's slots are spread out: stop.
+            unsigned long long pending = __ballot(active);
+#pragma unroll 1
+            for (int round = 0; round < kWaveGroups && pending != 0ull; ++round) {
+                const int leader = __builtin_ctzll(pending);
+                const uint32_t leader_slot = __builtin_amdgcn_readlane(slot[r], leader);
+                const bool in_group = miss && slot[r] == leader_slot;
+                const unsigned long long members = __ballot(in_group);
+                if (__popcll(members) < kMinWaveGroup) break;
+                const float s0 = lane_value(wave_sum_to_last_lane(in_group ? x0 : 0.0f), 63);
+                const float s1 = lane_value(wave_sum_to_last_lane(in_group ? x1 : 0.0f), 63);
+                const bool is_leader = static_cast<int>(threadIdx.x & 63) == leader;
+                x0 = is_leader ? s0 : x0;
+                x1 = is_leader ? s1 : x1;
+                miss = miss && (!in_group || is_leader);
+                hits += __popcll(members) - 1;  // absorbed without touching the cache
+                pending &= ~members;
             }
             bool found = false;
             if (miss) {
