@@ -131,9 +131,11 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
     float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
+    bool streaming = false;
     for (int t = 0; t < kScatterTiles; ++t) {
         const int64_t tile_base = (static_cast<int64_t>(blockIdx.x) * kScatterTiles + t) * kScatterBlock;
         if (tile_base >= n_points) break;
+        if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, blockIdx.x, t);
         const bool active = tile_base + threadIdx.x < n_points;
         const int nn = active ? static_cast<int>(tile_base) + threadIdx.x : n_points - 1;
         const float g0 = g0p[nn], g1 = g1p[nn];
@@ -145,11 +147,11 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
             PENC_INDEX(r);
             slot[r] = to_slot(h[r], capacity, cap_mask);
         });
-        const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t), slot,
-                                              w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
+        const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t),
+                                              streaming, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
         if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
     }
-    scatter_end(state, level_grad, bins, blockIdx.x);
+    scatter_end(state, level_grad, bins, blockIdx.x, streaming);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -229,9 +231,11 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
     const float* sf = scale_factor + lvl * D;
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
+    bool streaming = false;
     for (int t = 0; t < kScatterTiles; ++t) {
         const int64_t tile_base = (static_cast<int64_t>(blockIdx.x) * kScatterTiles + t) * kScatterBlock;
         if (tile_base >= n_points) break;
+        if (kTableGrad && live && !streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, blockIdx.x, t);
         const bool active = tile_base + threadIdx.x < n_points;
         const int n = static_cast<int>(tile_base) + threadIdx.x;
         const int nn = active ? n : n_points - 1;
@@ -258,7 +262,7 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
             if constexpr (kTableGrad) {
                 const float g0 = g0p[nn], g1 = g1p[nn];
                 const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t),
-                                                      slot, wr * g0, wr * g1);
+                                                      streaming, slot, wr * g0, wr * g1);
                 if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
             }
         }
@@ -268,7 +272,7 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
             o[n_points] = gg1;
         }
     }
-    if (kTableGrad && live) scatter_end(state, level_grad, bins, blockIdx.x);
+    if (kTableGrad && live) scatter_end(state, level_grad, bins, blockIdx.x, streaming);
 }
 
 // ------------------------------------------------------------------------------------------

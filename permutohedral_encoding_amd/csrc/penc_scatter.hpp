@@ -19,7 +19,10 @@
 //      private segment in every bin, so appending costs one LDS counter increment and one
 //      store); a second kernel (bin_reduce_kernel) reads each bin back coalesced, sums it in
 //      LDS (fp64), and adds the range into the gradient with coalesced read-modify-writes.  This
-//      turns the random scatter of the fine levels into streaming traffic.
+//      turns the random scatter of the fine levels into streaming traffic.  Once a workgroup has
+//      seen that its cache does not hit at a level, it gives the cache's LDS to its wavefronts as
+//      staging space: each wave sorts the records of a tile by bin there, so that records of one
+//      bin leave in runs of consecutive addresses instead of one 12-byte store each.
 //   3. Direct global atomics, with the two features of a slot in one instruction (lane pairs),
 //      for whatever is left: no workspace, capacity too large for binning, or a full bin.
 // The result never depends on a stage hitting: every stage falls through to the next.
@@ -39,6 +42,9 @@ constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
 constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
+constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space
+constexpr int kStageChunk = 4;         // vertices per thread a wave sorts by bin in one go (256 records)
+constexpr int kStageBins = 64;         // a wave counts one bin per lane: staging needs n_bins <= 64
 constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
 constexpr int kMaxBins = 512;          // bins per level; capacities above kMaxBins*kBinSlots (2^22) are not binned
@@ -98,6 +104,28 @@ __device__ __forceinline__ float wave_sum_to_last_lane(float v) {
 // The value `v` has in lane `lane` (wave-uniform index), broadcast to all lanes.
 __device__ __forceinline__ float lane_value(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Exclusive prefix sum over the 64 lanes of a wavefront; `total` is the sum of all lanes.
+__device__ __forceinline__ uint32_t wave_exclusive_scan(uint32_t v, uint32_t& total) {
+    // row_shr:1,2,4,8 scan each row of 16 (lanes shifted in from outside the row read 0);
+    // row_bcast:15 adds the total of rows 0 and 2 to rows 1 and 3, row_bcast:31 that of rows 0-1 to rows 2-3
+    int s = static_cast<int>(v);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x111, 0xf, 0xf, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x112, 0xf, 0xf, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x114, 0xf, 0xf, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x118, 0xf, 0xf, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x142, 0xa, 0xf, true);
+    s += __builtin_amdgcn_update_dpp(0, s, 0x143, 0xc, 0xf, true);
+    total = static_cast<uint32_t>(__builtin_amdgcn_readlane(s, 63));
+    return static_cast<uint32_t>(s) - v;
+}
+
+// Orders the LDS accesses of one wavefront: what its lanes wrote before is visible to all of them
+// after (LDS executes a wave's instructions in order; this keeps the compiler from reordering them).
+__device__ __forceinline__ void wave_lds_fence() {
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 }
 
 // Stage 3.  Lanes are paired (2p, 2p+1): first both lanes of a pair add the two features of the
@@ -189,15 +217,95 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
 }
 static_assert(kCacheLines == 1 << 11, "cache_find derives its second line from the top 11 bits of a product");
 
+// Stage 2 for a whole tile once the workgroup streams (see scatter_stream_switch): the cache's LDS
+// is staging space, a 4 KiB slice per wave.  For kStageChunk vertices per thread at a time, the wave
+// counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
+// bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
+// its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
+// Needs bins.n_bins <= kStageBins; all 64 lanes of the wave must call it together.
+template <int D>
+__device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+                                            uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
+                                            fvec<D + 1> a1) {
+    constexpr int kWaves = kScatterBlock / 64;
+    static_assert(kCacheLines / kWaves >= 3 * 64, "three 64-entry arrays per wave live in the tag array");
+    static_assert(sizeof(c.val) / kWaves >= kStageChunk * 64 * sizeof(uint4), "staging slice of a wave");
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    uint32_t* count = reinterpret_cast<uint32_t*>(c.tag) + wave * (kCacheLines / kWaves);  // records per bin
+    uint32_t* offset = count + 64;  // where a bin's run starts in the wave's slice
+    uint32_t* base = count + 128;   // where it starts in the workgroup's segment of that bin
+    uint4* stage = reinterpret_cast<uint4*>(c.val) + wave * (kStageChunk * 64);
+    constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
+    static_for<kChunks>(PENC_BODY(chunk) {
+        PENC_INDEX(chunk);
+        constexpr int kFirst = chunk * kStageChunk;
+        constexpr int kCount = D + 1 - kFirst < kStageChunk ? D + 1 - kFirst : kStageChunk;
+        count[lane] = 0u;
+        wave_lds_fence();
+        uvec<kStageChunk> place = 0u;  // rank of each record within its bin's run
+        static_for<kCount>(PENC_BODY(j) {
+            PENC_INDEX(j);
+            if (active) place[j] = atomicAdd(&count[slot[kFirst + j] >> kBinSlotsLog2], 1u);
+        });
+        wave_lds_fence();
+        const uint32_t mine = count[lane];
+        uint32_t total;
+        offset[lane] = wave_exclusive_scan(mine, total);
+        base[lane] = mine != 0u ? atomicAdd(&c.bin_count[lane], mine) : 0u;
+        wave_lds_fence();
+        static_for<kCount>(PENC_BODY(j) {
+            PENC_INDEX(j);
+            if (active) {
+                const uint32_t b = slot[kFirst + j] >> kBinSlotsLog2;
+                // copies first: a bit cast applied directly to a vector element reads element 0
+                const float v0 = a0[kFirst + j], v1 = a1[kFirst + j];
+                uint4 e;
+                e.x = slot[kFirst + j];
+                e.y = __builtin_bit_cast(uint32_t, v0);
+                e.z = __builtin_bit_cast(uint32_t, v1);
+                e.w = base[b] + place[j];
+                stage[offset[b] + place[j]] = e;
+            }
+        });
+        wave_lds_fence();
+        static_for<kCount>(PENC_BODY(j) {
+            PENC_INDEX(j);
+            const uint32_t i = j * 64 + lane;
+            bool spill = false;
+            uint4 e = {0u, 0u, 0u, 0u};
+            if (i < total) {
+                e = stage[i];
+                if (e.w < bins.segment_capacity) {
+                    BinRecord rec;
+                    rec.slot_in_bin = e.x & (kBinSlots - 1);
+                    rec.a0 = __builtin_bit_cast(float, e.y);
+                    rec.a1 = __builtin_bit_cast(float, e.z);
+                    const size_t segment = static_cast<size_t>(e.x >> kBinSlotsLog2) * bins.n_groups + group;
+                    bins.records[segment * bins.segment_capacity + e.w] = rec;
+                } else {
+                    spill = true;  // the segment is full: stage 3
+                }
+            }
+            if (__any(spill))
+                global_add_pairs(level_grad, spill, e.x, __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
+        });
+        wave_lds_fence();
+    });
+}
+
 // One tile's D+1 contributions per thread through stages 1-3.  All 64 lanes of every wave must
 // call it together; `active` is false for lanes that carry no point (tail of the last tile), which
 // only take part in the wave-wide steps.  `use_cache` (wave-uniform) is false once the workgroup
-// has seen that the cache does not hit at this level; the return value is the number of hits of
-// this wave in this tile.
+// has seen that the cache does not hit at this level; `streaming` is what scatter_stream_switch
+// returned.  The return value is the number of hits of this wave in this tile.
 template <int D>
 __device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
-                                                 uint32_t group, bool active, bool use_cache, uvec<D + 1> slot,
-                                                 fvec<D + 1> a0, fvec<D + 1> a1) {
+                                                 uint32_t group, bool active, bool use_cache, bool streaming,
+                                                 uvec<D + 1> slot, fvec<D + 1> a0, fvec<D + 1> a1) {
+    if (streaming) {
+        stream_tile<D>(c, level_grad, bins, group, active, slot, a0, a1);
+        return 0u;
+    }
     uint32_t hits = 0;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
@@ -251,11 +359,9 @@ __device__ __forceinline__ bool cache_pays(const ScatterState& c, int tiles_done
     return tiles_done == 0 || c.hits * 8u >= static_cast<uint32_t>(tiles_done) * kScatterBlock * (D + 1);
 }
 
-// After the last tile: flushes the accumulate cache (through the bins when there are any) and
-// publishes how many records this workgroup left in each bin.  Call once, by all threads.
-__device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+// Sends every line of the accumulate cache on to stage 2 (or 3).  By all threads, between barriers.
+__device__ __forceinline__ void cache_flush(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
                                             uint32_t group) {
-    __syncthreads();
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         const int owner = c.tag[e];
         if (owner != -1) {
@@ -268,6 +374,31 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
             }
         }
     }
+}
+
+// Before tile `tile` (all threads call it, with the same arguments): decides for the whole
+// workgroup whether to give up the accumulate cache for good and use its LDS as staging space
+// (stream_tile).  Returns true from then on; the cache's contents have been flushed by then.
+template <int D>
+__device__ __forceinline__ bool scatter_stream_switch(ScatterState& c, float* __restrict__ level_grad,
+                                                      const BinTarget& bins, uint32_t group, int tile) {
+    if (tile != kStreamDecisionTile || bins.records == nullptr || bins.n_bins > kStageBins) return false;
+    __syncthreads();  // the hits of the tiles so far are in
+    const bool stream = !cache_pays<D>(c, tile);
+    __syncthreads();  // everyone has read the count before a fast wave adds the next tile's hits
+    if (!stream) return false;
+    cache_flush(c, level_grad, bins, group);
+    __syncthreads();
+    return true;
+}
+
+// After the last tile: flushes the accumulate cache (through the bins when there are any; a
+// streaming workgroup has none left) and publishes how many records this workgroup left in each
+// bin.  Call once, by all threads.
+__device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+                                            uint32_t group, bool streaming) {
+    __syncthreads();
+    if (!streaming) cache_flush(c, level_grad, bins, group);
     if (bins.records == nullptr) return;
     __syncthreads();
     for (uint32_t b = threadIdx.x; b < bins.n_bins; b += kScatterBlock) {
