@@ -131,15 +131,26 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
     float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
+    // A tile's inputs are fetched one tile ahead: their latency then overlaps the previous tile's
+    // scatter instead of stalling the wave at the top of every iteration.
+    const int64_t group_base = static_cast<int64_t>(blockIdx.x) * kGroupPoints;
+    const auto point_of = [&](int t) {  // the point this thread handles in tile t (clamped: the tail re-reads the last point)
+        const int64_t n = group_base + static_cast<int64_t>(t) * kScatterBlock + threadIdx.x;
+        return static_cast<int>(n < n_points ? n : n_points - 1);
+    };
+    int nn = point_of(0);
+    fvec<D> pos = load_point<D>(positions, nn);
+    float g0 = g0p[nn], g1 = g1p[nn];
     bool streaming = false;
     for (int t = 0; t < kScatterTiles; ++t) {
-        const int64_t tile_base = (static_cast<int64_t>(blockIdx.x) * kScatterTiles + t) * kScatterBlock;
+        const int64_t tile_base = group_base + static_cast<int64_t>(t) * kScatterBlock;
         if (tile_base >= n_points) break;
-        if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, blockIdx.x, t);
         const bool active = tile_base + threadIdx.x < n_points;
-        const int nn = active ? static_cast<int>(tile_base) + threadIdx.x : n_points - 1;
-        const float g0 = g0p[nn], g1 = g1p[nn];
-        const Located<D> s = locate<D>(load_point<D>(positions, nn), random_shift + level * D, scale_factor + level * D);
+        const int nn_next = point_of(t + 1);
+        const fvec<D> pos_next = load_point<D>(positions, nn_next);
+        const float g0_next = g0p[nn_next], g1_next = g1p[nn_next];
+        if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, blockIdx.x, t);
+        const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
         const fvec<D + 1> w = barycentric<D>(s.rank, s.delta) * w_level;
         uvec<D + 1> slot;
@@ -150,6 +161,9 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
         const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t),
                                               streaming, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
         if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
+        pos = pos_next;
+        g0 = g0_next;
+        g1 = g1_next;
     }
     scatter_end(state, level_grad, bins, blockIdx.x, streaming);
 }
@@ -416,6 +430,11 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, void*
         if (bytes < segments * (sizeof(uint32_t) + 16 * sizeof(BinRecord))) return p;
         cap = static_cast<uint32_t>((bytes / segments - sizeof(uint32_t)) / sizeof(BinRecord));
     }
+    // the scattering kernel indexes a level's records with 32 bits
+    if (segments * cap > 0xFFFFFFFFull) {
+        cap = static_cast<uint32_t>(0xFFFFFFFFull / segments);
+        if (cap < 16) return p;
+    }
     const size_t fit = bytes / bin_bytes_per_level(n_bins, n_groups, cap);
     p.levels_per_pass = static_cast<int>(fit < static_cast<size_t>(levels) ? fit : static_cast<size_t>(levels));
     p.target.n_bins = n_bins;
@@ -430,9 +449,17 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, void*
 
 // Running consecutive passes on two streams (scatter pass p+1 while pass p is reduced) was tried and
 // measured 10-15% slower than one pass over all levels on one stream; hence a single stream.
+constexpr unsigned kReduceWorkgroupsWanted = 512;  // two per compute unit
+constexpr unsigned kMaxReduceSplits = 16;
+
 inline int reduce_bins(const BinPlan& p, const float* window, int first_level, int n_levels_in_pass, int capacity,
                        float* table_grad, hipStream_t st) {
-    hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass), dim3(kReduceBlock), 0, st,
+    // enough workgroups for every compute unit, by letting several share a bin when bins*levels is small
+    const unsigned pairs = p.target.n_bins * static_cast<unsigned>(n_levels_in_pass);
+    unsigned splits = pairs >= kReduceWorkgroupsWanted ? 1u : (kReduceWorkgroupsWanted + pairs - 1) / pairs;
+    if (splits > p.target.n_groups) splits = p.target.n_groups;
+    if (splits > kMaxReduceSplits) splits = kMaxReduceSplits;
+    hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass, splits), dim3(kReduceBlock), 0, st,
                        p.target, window, static_cast<uint32_t>(capacity), table_grad, first_level);
     return check_launch();
 }

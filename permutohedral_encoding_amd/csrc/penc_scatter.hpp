@@ -39,7 +39,8 @@ constexpr int kBlock = 256;            // threads per workgroup of the gather-ty
 constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wavefronts share one accumulate cache)
 constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
 constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
-constexpr int kCacheLines = 2048;      // accumulate-cache lines per workgroup
+constexpr int kCacheLinesLog2 = 11;
+constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per workgroup
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
 constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space
@@ -196,6 +197,8 @@ __device__ __forceinline__ bool append_record(ScatterState& c, const BinTarget& 
 // loses several of them to collisions, and those are exactly the slots every wave keeps hitting.
 // Returns the line, or -1 when both candidates belong to other slots; `found` tells whether the
 // line already held the slot (a hit, as opposed to a claim).
+// (Spreading the lanes that share a slot over replicated sub-tables, instead of folding them in
+// registers first, was measured 30% slower on the coarse levels, and no faster on top of folding.)
 __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& found) {
     const int want = static_cast<int>(slot);
     int e = static_cast<int>(slot & (kCacheLines - 1));
@@ -211,30 +214,32 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
             owner = atomicCAS(&c.tag[e], -1, want);
             if (owner == -1 || owner == want) return e;
         }
-        e = static_cast<int>((slot * 0x9E3779B1u) >> (32 - 11)) & (kCacheLines - 1);
+        e = static_cast<int>((slot * 0x9E3779B1u) >> (32 - kCacheLinesLog2));
     }
     return -1;
 }
-static_assert(kCacheLines == 1 << 11, "cache_find derives its second line from the top 11 bits of a product");
 
 // Stage 2 for a whole tile once the workgroup streams (see scatter_stream_switch): the cache's LDS
 // is staging space, a 4 KiB slice per wave.  For kStageChunk vertices per thread at a time, the wave
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
 // its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
-// Needs bins.n_bins <= kStageBins; all 64 lanes of the wave must call it together.
+// Needs bins.n_bins <= kStageBins and a level's record array below 2^32 records (the host plans
+// for both); all 64 lanes of the wave must call it together.
 template <int D>
 __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
                                             uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
                                             fvec<D + 1> a1) {
     constexpr int kWaves = kScatterBlock / 64;
-    static_assert(kCacheLines / kWaves >= 3 * 64, "three 64-entry arrays per wave live in the tag array");
+    static_assert(kCacheLines / kWaves >= 4 * 64, "four 64-entry arrays per wave live in the tag array");
     static_assert(sizeof(c.val) / kWaves >= kStageChunk * 64 * sizeof(uint4), "staging slice of a wave");
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     uint32_t* count = reinterpret_cast<uint32_t*>(c.tag) + wave * (kCacheLines / kWaves);  // records per bin
     uint32_t* offset = count + 64;  // where a bin's run starts in the wave's slice
-    uint32_t* base = count + 128;   // where it starts in the workgroup's segment of that bin
+    uint32_t* start = count + 128;  // index of the run's first record in the level's record array
+    uint32_t* room = count + 192;   // records the workgroup's segment of the bin can still take
     uint4* stage = reinterpret_cast<uint4*>(c.val) + wave * (kStageChunk * 64);
+    constexpr uint32_t kNoRoom = 0xFFFFFFFFu;
     constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
     static_for<kChunks>(PENC_BODY(chunk) {
         PENC_INDEX(chunk);
@@ -248,10 +253,13 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
             if (active) place[j] = atomicAdd(&count[slot[kFirst + j] >> kBinSlotsLog2], 1u);
         });
         wave_lds_fence();
+        // lane b looks after bin b: one reservation and one index computation per bin, not per record
         const uint32_t mine = count[lane];
         uint32_t total;
         offset[lane] = wave_exclusive_scan(mine, total);
-        base[lane] = mine != 0u ? atomicAdd(&c.bin_count[lane], mine) : 0u;
+        const uint32_t taken = mine != 0u ? atomicAdd(&c.bin_count[lane], mine) : 0u;
+        start[lane] = (lane * bins.n_groups + group) * bins.segment_capacity + taken;
+        room[lane] = taken < bins.segment_capacity ? bins.segment_capacity - taken : 0u;
         wave_lds_fence();
         static_for<kCount>(PENC_BODY(j) {
             PENC_INDEX(j);
@@ -263,7 +271,7 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
                 e.x = slot[kFirst + j];
                 e.y = __builtin_bit_cast(uint32_t, v0);
                 e.z = __builtin_bit_cast(uint32_t, v1);
-                e.w = base[b] + place[j];
+                e.w = place[j] < room[b] ? start[b] + place[j] : kNoRoom;
                 stage[offset[b] + place[j]] = e;
             }
         });
@@ -275,13 +283,12 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
             uint4 e = {0u, 0u, 0u, 0u};
             if (i < total) {
                 e = stage[i];
-                if (e.w < bins.segment_capacity) {
+                if (e.w != kNoRoom) {
                     BinRecord rec;
                     rec.slot_in_bin = e.x & (kBinSlots - 1);
                     rec.a0 = __builtin_bit_cast(float, e.y);
                     rec.a1 = __builtin_bit_cast(float, e.z);
-                    const size_t segment = static_cast<size_t>(e.x >> kBinSlotsLog2) * bins.n_groups + group;
-                    bins.records[segment * bins.segment_capacity + e.w] = rec;
+                    bins.records[e.w] = rec;
                 } else {
                     spill = true;  // the segment is full: stage 3
                 }
@@ -407,13 +414,16 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
     }
 }
 
-// Second kernel of stage 2: one workgroup per (bin, level) sums the bin's records in LDS (fp64,
+// Second kernel of stage 2: a workgroup sums the records of one (bin, level) in LDS (fp64,
 // ds_add_f64: a few hot slots must not serialise the whole bin, which rules out a compare-and-swap
-// loop) and adds the bin's slot range into the gradient.  Each wavefront takes whole segments (one
-// per scattering workgroup), so its loads are contiguous; a segment's records are fetched four
-// wave-widths at a time so that several loads are in flight.  Nothing else touches the gradient
-// while this kernel runs (the scattering kernel before it has completed, and bins do not
-// overlap), so the final add is a plain coalesced read-modify-write.
+// loop) and adds the bin's slot range into the gradient.  gridDim.z workgroups share a bin, each
+// taking a contiguous range of the scattering workgroups' segments (a launch over few levels would
+// otherwise leave most of the chip idle).  Each wavefront takes whole segments, so its loads are
+// contiguous; a segment's records are fetched four wave-widths at a time so that several loads are
+// in flight.  With one workgroup per bin nothing else touches the bin's slots while this kernel
+// runs (the scattering kernel before it has completed, and bins do not overlap), so the final add is
+// a plain coalesced read-modify-write; workgroups that share a bin add with atomics (consecutive
+// addresses: one request per 64 bytes).
 __global__ void __launch_bounds__(kReduceBlock)
 bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity,
                   float* __restrict__ table_grad, int first_level) {
@@ -430,14 +440,17 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     constexpr uint32_t kWaves = kReduceBlock / 64;
     constexpr uint32_t kUnroll = 4;
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t per_split = (bins.n_groups + gridDim.z - 1) / gridDim.z;
+    const uint32_t group_begin = blockIdx.z * per_split;
+    const uint32_t group_end = group_begin + per_split < bins.n_groups ? group_begin + per_split : bins.n_groups;
     const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
     const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
-    // segments g = wave, wave + kWaves, ...; their record counts are fetched 64 at a time (one per
-    // lane) so that no segment has to wait for its own count
-    for (uint32_t g0 = wave; g0 < bins.n_groups; g0 += kWaves * 64) {
+    // segments g = group_begin + wave, + kWaves, ...; their record counts are fetched 64 at a time
+    // (one per lane) so that no segment has to wait for its own count
+    for (uint32_t g0 = group_begin + wave; g0 < group_end; g0 += kWaves * 64) {
         const uint32_t mine = g0 + lane * kWaves;
-        const uint32_t my_count = mine < bins.n_groups ? counts[mine] : 0u;
-        for (uint32_t k = 0; k < 64 && g0 + k * kWaves < bins.n_groups; ++k) {
+        const uint32_t my_count = mine < group_end ? counts[mine] : 0u;
+        for (uint32_t k = 0; k < 64 && g0 + k * kWaves < group_end; ++k) {
             const uint32_t count = __builtin_amdgcn_readlane(my_count, k);
             const BinRecord* seg = recs + static_cast<size_t>(g0 + k * kWaves) * bins.segment_capacity;
             for (uint32_t base = 0; base < count; base += 64 * kUnroll) {
@@ -460,13 +473,19 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     __syncthreads();
     float2* level_grad = reinterpret_cast<float2*>(table_grad + static_cast<size_t>(level) * capacity * 2);
     const uint32_t slot0 = bin << kBinSlotsLog2;
+    const bool alone = gridDim.z == 1;
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
         const double v0 = acc[s][0], v1 = acc[s][1];
         if ((v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity) {
-            float2 g = level_grad[slot0 + s];
-            g.x += static_cast<float>(v0);
-            g.y += static_cast<float>(v1);
-            level_grad[slot0 + s] = g;
+            if (alone) {
+                float2 g = level_grad[slot0 + s];
+                g.x += static_cast<float>(v0);
+                g.y += static_cast<float>(v1);
+                level_grad[slot0 + s] = g;
+            } else {
+                global_add(&level_grad[slot0 + s].x, static_cast<float>(v0));
+                global_add(&level_grad[slot0 + s].y, static_cast<float>(v1));
+            }
         }
     }
 }
