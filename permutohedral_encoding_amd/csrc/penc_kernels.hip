@@ -71,7 +71,9 @@ __device__ __forceinline__ Vertices<D> load_vertices(const float* __restrict__ l
 // thread (more loads in flight per lane: no gain, the kernel already runs at the rate this GPU
 // sustains for random 8-byte loads from a 2 MiB slice); walking the levels inside the thread with
 // the positions kept in registers (20% slower at 2^20 points, 3x slower at 2^16: fewer, longer
-// waves lose more than the re-read positions cost).
+// waves lose more than the re-read positions cost); interleaving workgroups of a coarse
+// (compute-bound) and a fine (gather-bound) level, which takes the fine level's slice out of L2
+// (30% slower).
 
 template <int D>
 __global__ void __launch_bounds__(kBlock)
@@ -118,22 +120,27 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 
 template <int D>
 __global__ void __launch_bounds__(kScatterBlock)
-backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t cap_mask,
+backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t capacity, uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
                       const float* __restrict__ grad_sliced, float* __restrict__ table_grad, BinTarget pass_bins) {
     __shared__ ScatterState state;
-    const int level = first_level + blockIdx.y;
+    // blockIdx.x = group * levels + level: neighbouring workgroups take the same points at different
+    // levels, so the points are fetched from memory once, and compute-bound coarse levels and
+    // store-bound fine levels share the chip at all times (this kernel never reads the table, so
+    // there is no slice to keep cache-resident by running a level at a time)
+    const uint32_t level_in_pass = blockIdx.x % n_pass_levels, group = blockIdx.x / n_pass_levels;
+    const int level = first_level + level_in_pass;
     const float w_level = window[level];
     if (w_level == 0.0f) return;
     scatter_begin(state);
-    const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
+    const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
     // A tile's inputs are fetched one tile ahead: their latency then overlaps the previous tile's
     // scatter instead of stalling the wave at the top of every iteration.
-    const int64_t group_base = static_cast<int64_t>(blockIdx.x) * kGroupPoints;
+    const int64_t group_base = static_cast<int64_t>(group) * kGroupPoints;
     const auto point_of = [&](int t) {  // the point this thread handles in tile t (clamped: the tail re-reads the last point)
         const int64_t n = group_base + static_cast<int64_t>(t) * kScatterBlock + threadIdx.x;
         return static_cast<int>(n < n_points ? n : n_points - 1);
@@ -149,7 +156,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
         const int nn_next = point_of(t + 1);
         const fvec<D> pos_next = load_point<D>(positions, nn_next);
         const float g0_next = g0p[nn_next], g1_next = g1p[nn_next];
-        if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, blockIdx.x, t);
+        if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
         const fvec<D + 1> w = barycentric<D>(s.rank, s.delta) * w_level;
@@ -158,14 +165,14 @@ backward_table_kernel(int n_points, int first_level, uint32_t capacity, uint32_t
             PENC_INDEX(r);
             slot[r] = to_slot(h[r], capacity, cap_mask);
         });
-        const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t),
+        const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
                                               streaming, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
         if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
         pos = pos_next;
         g0 = g0_next;
         g1 = g1_next;
     }
-    scatter_end(state, level_grad, bins, blockIdx.x, streaming);
+    scatter_end(state, level_grad, bins, group, streaming);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -232,14 +239,17 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
                        const float* __restrict__ grad_sliced, float* __restrict__ table_grad,
                        float* __restrict__ grad_grad_sliced, BinTarget pass_bins) {
     __shared__ ScatterState state;
-    const int level = first_level + blockIdx.y;
+    // a level at a time (blockIdx.y), unlike backward_table_kernel: this kernel gathers from the
+    // table, and interleaving levels was measured equal to 13% slower (the slices fall out of L2)
+    const uint32_t level_in_pass = blockIdx.y, group = blockIdx.x;
+    const int level = first_level + level_in_pass;
     const bool extra_level = level >= n_levels;  // concat levels: zeros (:1290-1295)
     const float w_level = extra_level ? 0.0f : window[level];
     const bool live = w_level != 0.0f;
     if (!live && !kGradGrad) return;
     if (kTableGrad && live) scatter_begin(state);
     const int lvl = extra_level ? 0 : level;
-    const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
+    const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     float* level_grad = kTableGrad ? table_grad + static_cast<size_t>(lvl) * capacity * 2 : nullptr;
     const float* level_table = table + static_cast<size_t>(lvl) * capacity * 2;
     const float* sf = scale_factor + lvl * D;
@@ -247,9 +257,9 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
     const float* g1p = g0p + n_points;
     bool streaming = false;
     for (int t = 0; t < kScatterTiles; ++t) {
-        const int64_t tile_base = (static_cast<int64_t>(blockIdx.x) * kScatterTiles + t) * kScatterBlock;
+        const int64_t tile_base = (static_cast<int64_t>(group) * kScatterTiles + t) * kScatterBlock;
         if (tile_base >= n_points) break;
-        if (kTableGrad && live && !streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, blockIdx.x, t);
+        if (kTableGrad && live && !streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
         const bool active = tile_base + threadIdx.x < n_points;
         const int n = static_cast<int>(tile_base) + threadIdx.x;
         const int nn = active ? n : n_points - 1;
@@ -275,7 +285,7 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
             }
             if constexpr (kTableGrad) {
                 const float g0 = g0p[nn], g1 = g1p[nn];
-                const uint32_t hits = scatter_tile<D>(state, level_grad, bins, blockIdx.x, active, cache_pays<D>(state, t),
+                const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
                                                       streaming, slot, wr * g0, wr * g1);
                 if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
             }
@@ -286,7 +296,7 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
             o[n_points] = gg1;
         }
     }
-    if (kTableGrad && live) scatter_end(state, level_grad, bins, blockIdx.x, streaming);
+    if (kTableGrad && live) scatter_end(state, level_grad, bins, group, streaming);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -568,9 +578,9 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
         const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
         for (int first = 0; first < nr_levels; first += per_pass) {
             const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
-            const dim3 grid(scatter_groups(nr_positions), count);
+            const dim3 grid(scatter_groups(nr_positions) * static_cast<unsigned>(count));
             PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD>), grid, dim3(kScatterBlock), 0, st, n,
-                                                        first, cap, mask, positions, scale_factor, random_shift,
+                                                        first, static_cast<uint32_t>(count), cap, mask, positions, scale_factor, random_shift,
                                                         anneal_window, grad_sliced_values, lattice_values_grad,
                                                         plan.target));
             if (int rc = check_launch()) return rc;
