@@ -125,11 +125,15 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
                       const float* __restrict__ random_shift, const float* __restrict__ window,
                       const float* __restrict__ grad_sliced, float* __restrict__ table_grad, BinTarget pass_bins) {
     __shared__ ScatterState state;
-    // blockIdx.x = group * levels + level: neighbouring workgroups take the same points at different
-    // levels, so the points are fetched from memory once, and compute-bound coarse levels and
-    // store-bound fine levels share the chip at all times (this kernel never reads the table, so
-    // there is no slice to keep cache-resident by running a level at a time)
-    const uint32_t level_in_pass = blockIdx.x % n_pass_levels, group = blockIdx.x / n_pass_levels;
+    // Workgroups are dealt round-robin to the kXcds dies, each with an L2 of its own.  The j-th
+    // workgroup of a die takes level j % levels of one group of points: a die works through all
+    // levels of a group before the next group, so the points are fetched from memory once, and
+    // compute-bound coarse levels and store-bound fine levels share the chip at all times (this
+    // kernel never reads the table: there is no slice to keep cache-resident by running a level at
+    // a time).
+    const uint32_t die = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
+    const uint32_t level_in_pass = j % n_pass_levels, group = (j / n_pass_levels) * kXcds + die;
+    if (static_cast<int64_t>(group) * kGroupPoints >= n_points) return;
     const int level = first_level + level_in_pass;
     const float w_level = window[level];
     if (w_level == 0.0f) return;
@@ -578,7 +582,8 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
         const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
         for (int first = 0; first < nr_levels; first += per_pass) {
             const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
-            const dim3 grid(scatter_groups(nr_positions) * static_cast<unsigned>(count));
+            const unsigned padded_groups = (scatter_groups(nr_positions) + kXcds - 1) / kXcds * kXcds;
+            const dim3 grid(padded_groups * static_cast<unsigned>(count));
             PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD>), grid, dim3(kScatterBlock), 0, st, n,
                                                         first, static_cast<uint32_t>(count), cap, mask, positions, scale_factor, random_shift,
                                                         anneal_window, grad_sliced_values, lattice_values_grad,

@@ -35,6 +35,7 @@
 
 namespace penc {
 
+constexpr int kXcds = 8;               // accelerator dies (XCDs) of the chip; workgroup i runs on die i % kXcds
 constexpr int kBlock = 256;            // threads per workgroup of the gather-type kernels (4 wavefronts)
 constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wavefronts share one accumulate cache)
 constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
@@ -419,8 +420,7 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
 // loop) and adds the bin's slot range into the gradient.  gridDim.z workgroups share a bin, each
 // taking a contiguous range of the scattering workgroups' segments (a launch over few levels would
 // otherwise leave most of the chip idle).  Each wavefront takes whole segments, so its loads are
-// contiguous; a segment's records are fetched four wave-widths at a time so that several loads are
-// in flight.  With one workgroup per bin nothing else touches the bin's slots while this kernel
+// contiguous.  With one workgroup per bin nothing else touches the bin's slots while this kernel
 // runs (the scattering kernel before it has completed, and bins do not overlap), so the final add is
 // a plain coalesced read-modify-write; workgroups that share a bin add with atomics (consecutive
 // addresses: one request per 64 bytes).
@@ -429,9 +429,12 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
                   float* __restrict__ table_grad, int first_level) {
     __shared__ double acc[kBinSlots][2];
     const uint32_t bin = blockIdx.x;
-    const int level = first_level + blockIdx.y;
+    // last level first: with the usual coarse-to-fine level list the bins with the most records are
+    // started first and the nearly empty ones fill the tail of the launch
+    const uint32_t level_in_pass = gridDim.y - 1 - blockIdx.y;
+    const int level = first_level + level_in_pass;
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
-    const BinTarget bins = bins_of_level(pass_bins, blockIdx.y);
+    const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
         acc[s][0] = 0.0;
         acc[s][1] = 0.0;
@@ -446,28 +449,47 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
     const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
     // segments g = group_begin + wave, + kWaves, ...; their record counts are fetched 64 at a time
-    // (one per lane) so that no segment has to wait for its own count
+    // (one per lane) so that no segment has to wait for its own count.  The records are walked in
+    // chunks of kUnroll wave-widths, and the next chunk's loads are issued before the current
+    // chunk's LDS atomics, so a wave always has loads in flight.
+    constexpr uint32_t kChunk = 64 * kUnroll;
     for (uint32_t g0 = group_begin + wave; g0 < group_end; g0 += kWaves * 64) {
         const uint32_t mine = g0 + lane * kWaves;
         const uint32_t my_count = mine < group_end ? counts[mine] : 0u;
-        for (uint32_t k = 0; k < 64 && g0 + k * kWaves < group_end; ++k) {
-            const uint32_t count = __builtin_amdgcn_readlane(my_count, k);
+        const uint32_t n_segments = (group_end - g0 + kWaves - 1) / kWaves < 64u ? (group_end - g0 + kWaves - 1) / kWaves : 64u;
+        const auto count_of = [&](uint32_t k) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(my_count, k)); };
+        const auto fetch = [&](uint32_t k, uint32_t base, BinRecord (&rec)[kUnroll]) {
+            const uint32_t count = count_of(k);
             const BinRecord* seg = recs + static_cast<size_t>(g0 + k * kWaves) * bins.segment_capacity;
-            for (uint32_t base = 0; base < count; base += 64 * kUnroll) {
-                BinRecord rec[kUnroll];
 #pragma unroll
-                for (uint32_t u = 0; u < kUnroll; ++u) {
-                    const uint32_t i = base + u * 64 + lane;
-                    rec[u] = seg[i < count ? i : 0];
+            for (uint32_t u = 0; u < kUnroll; ++u) {
+                const uint32_t i = base + u * 64 + lane;
+                rec[u] = seg[i < count ? i : 0];
+            }
+        };
+        uint32_t k = 0, base = 0;
+        while (k < n_segments && count_of(k) == 0u) ++k;
+        BinRecord cur[kUnroll], next[kUnroll];
+        if (k < n_segments) fetch(k, base, cur);
+        while (k < n_segments) {
+            const uint32_t count = count_of(k);
+            uint32_t next_k = k, next_base = base + kChunk;
+            if (next_base >= count) {
+                next_base = 0;
+                do ++next_k; while (next_k < n_segments && count_of(next_k) == 0u);
+            }
+            if (next_k < n_segments) fetch(next_k, next_base, next);
+#pragma unroll
+            for (uint32_t u = 0; u < kUnroll; ++u)
+                if (base + u * 64 + lane < count) {
+                    double* cell = acc[cur[u].slot_in_bin];
+                    __hip_atomic_fetch_add(cell, static_cast<double>(cur[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(cell + 1, static_cast<double>(cur[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
 #pragma unroll
-                for (uint32_t u = 0; u < kUnroll; ++u)
-                    if (base + u * 64 + lane < count) {
-                        double* cell = acc[rec[u].slot_in_bin];
-                        __hip_atomic_fetch_add(cell, static_cast<double>(rec[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                        __hip_atomic_fetch_add(cell + 1, static_cast<double>(rec[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    }
-            }
+            for (uint32_t u = 0; u < kUnroll; ++u) cur[u] = next[u];
+            k = next_k;
+            base = next_base;
         }
     }
     __syncthreads();
