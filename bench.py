@@ -11,7 +11,8 @@ every input already resident in HBM.  Prints ONE JSON line:
   cpu_baseline the CPU oracle (a scalar-code OpenMP port of the reference kernels) timed on this
                machine's host cores on a bounded sample of the same workload
   probes       measured streaming / random-gather / random-atomic rates of this GPU, which are what
-               the table traffic is really bounded by
+               the table traffic is really bounded by; hbm_traffic_rate relates the measured HBM
+               bytes of each phase to them
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu]
 """
@@ -244,18 +245,17 @@ def main():
     }
     if not args.no_probes:
         result["probes"] = run_probes(torch, _native, cap, n, d + 1)
-        pr = result["probes"]
-        # What the table traffic alone would take if every one of the N*L*(D+1) slot accesses of each
-        # table-touching phase (gather or scatter alike) ran at the measured random 8-byte gather rate,
-        # plus the streaming traffic at the measured copy rate.
-        table_phases = sum(1 for name, _ in phases if name == "forward" or (name == "backward" and (want_table or want_pos))
-                           or name == "double_backward") + (1 if ("backward", backward) in phases and want_table and want_pos else 0)
-        bound_s = table_phases * w.point_levels * (d + 1) / (pr["gather_Gacc_per_s"] * 1e9)
-        stream_bytes = sum(phase_bytes[name] - 8 * (d + 1) * (2 if name == "double_backward" else 1) for name, _ in phases) * w.point_levels
-        bound_s += max(stream_bytes, 0.0) / (pr["copy_GBps"] * 1e9)
-        result["measured_roofline"] = {"bound_ms": bound_s * 1e3, "frac": bound_s * 1e3 / ms_per_step,
-                                       "note": "every table slot access at the probe's random-gather rate + streaming at "
-                                               "the probe's copy rate; frac = bound / measured step"}
+        # How fast the HBM traffic each phase really makes (hardware byte counters, scaled by the copy
+        # probe, from profiles/) is moved, next to the rate the copy probe reaches for pure streaming.
+        if os.path.exists(traffic_file):
+            with open(traffic_file) as f:
+                per_phase = json.load(f).get(w.name, {})
+            result["hbm_traffic_rate"] = {
+                "GBps": {k: per_phase[k] / (phase_ms[k] * 1e-3) / 1e9 for k in phase_ms if k in per_phase},
+                "copy_probe_GBps": result["probes"]["copy_GBps"],
+                "note": "measured HBM bytes per launch / measured phase time; the forward is bound by random 8-byte "
+                        "gathers (see probes.gather_Gacc_per_s), the table backward by streaming its slot-range records",
+            }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w, inputs, args.cpu_sample)
     print(json.dumps(result))
