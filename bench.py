@@ -245,6 +245,20 @@ def main():
     }
     if not args.no_probes:
         result["probes"] = run_probes(torch, _native, cap, n, d + 1)
+        pr = result["probes"]
+        # The measured L2/MALL gather roofline: what the step would take if every one of the
+        # N*L*(D+1) slot accesses of each table-touching phase (gather or scatter alike) ran at the
+        # measured random 8-byte gather rate, plus the streaming traffic at the measured copy rate.
+        # frac can exceed 1: the coarse levels hit caches better than the probe's uniform indices, and
+        # the binned table backward replaces random slot accesses by streamed records.
+        table_phases = sum(1 for name, _ in phases if name == "forward" or (name == "backward" and (want_table or want_pos))
+                           or name == "double_backward") + (1 if ("backward", backward) in phases and want_table and want_pos else 0)
+        bound_s = table_phases * w.point_levels * (d + 1) / (pr["gather_Gacc_per_s"] * 1e9)
+        stream_bytes = sum(phase_bytes[name] - 8 * (d + 1) * (2 if name == "double_backward" else 1) for name, _ in phases) * w.point_levels
+        bound_s += max(stream_bytes, 0.0) / (pr["copy_GBps"] * 1e9)
+        result["measured_roofline"] = {"bound_ms": bound_s * 1e3, "frac": bound_s * 1e3 / ms_per_step,
+                                       "note": "every table slot access at the probe's random-gather rate + streaming at "
+                                               "the probe's copy rate; frac = bound / measured step"}
         # How fast the HBM traffic each phase really makes (hardware byte counters, scaled by the copy
         # probe, from profiles/) is moved, next to the rate the copy probe reaches for pure streaming.
         if os.path.exists(traffic_file):

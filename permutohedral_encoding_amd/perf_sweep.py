@@ -1,0 +1,88 @@
+"""Module-level throughput sweep over the input dimension, in points per second.
+
+Follows the measurement protocol of the reference's performance script
+(``examples/performance.py:59-183``): 2^19 points uniform in [-0.5, 0.5]^d, 24 levels, 2 features
+per level, capacity 2^18, scales geomspace(1, 1e-4); every iteration is bracketed by a device
+synchronisation and timed with ``perf_counter``; 300 iterations of which the first 10 are discarded;
+throughput = points / second, averaged over the kept iterations.  Three modes:
+
+  inference        module forward under no_grad
+  train_table      forward, loss ((pred-10)^2).mean(), zero_grad, backward, AdamW step on the table
+  train_table_pos  the same with points that require a gradient
+
+Unlike the kernel benchmark (``bench.py``) these figures include everything a user of the module
+pays: output allocation, the loss, the gradient layout change and the optimiser walking the whole
+table.
+
+    python -m permutohedral_encoding_amd.perf_sweep [--dims 2 3 4 5 6] [--points 524288] [--iters 300]
+"""
+import argparse
+import json
+import time
+
+import numpy as np
+import torch
+
+from .modules import PermutoEncoding
+
+
+def _timed(step, nr_points, iters, warmup):
+    kept = []
+    for it in range(iters):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if it > warmup:
+            kept.append(nr_points / dt)
+    return float(np.mean(kept))
+
+
+def measure(pos_dim, nr_points, iters, warmup, levels=24, log2_capacity=18):
+    torch.manual_seed(0)
+    enc = PermutoEncoding(pos_dim, 1 << log2_capacity, levels, 2, np.geomspace(1.0, 1e-4, num=levels))
+    opt = torch.optim.AdamW(enc.parameters(), amsgrad=False, betas=(0.9, 0.99), eps=1e-15, weight_decay=0.0, lr=1e-3)
+    pts = torch.rand(nr_points, pos_dim, device="cuda") - 0.5
+    pts_grad = pts.clone().requires_grad_(True)
+
+    def inference():
+        with torch.no_grad():
+            enc(pts)
+
+    def train(points):
+        pred = enc(points)
+        loss = ((pred - 10) ** 2).mean()
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+
+    enc.eval()
+    res = {"pos_dim": pos_dim, "points": nr_points, "inference": _timed(inference, nr_points, iters, warmup)}
+    enc.train()
+    res["train_table"] = _timed(lambda: train(pts), nr_points, iters, warmup)
+    res["train_table_pos"] = _timed(lambda: train(pts_grad), nr_points, iters, warmup)
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--dims", type=int, nargs="+", default=[2, 3, 4, 5, 6])
+    ap.add_argument("--points", type=int, default=1 << 19)
+    ap.add_argument("--iters", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=10)
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        raise SystemExit("perf_sweep: no GPU visible; the encoding has no CPU path")
+    print("| pos_dim | inference (points/s) | training, table grad (points/s) | training, table + position grad (points/s) |")
+    print("|---|---|---|---|")
+    rows = []
+    for d in args.dims:
+        r = measure(d, args.points, args.iters, args.warmup)
+        rows.append(r)
+        print(f"| {d} | {r['inference']:.3g} | {r['train_table']:.3g} | {r['train_table_pos']:.3g} |", flush=True)
+    print(json.dumps(rows))
+
+
+if __name__ == "__main__":
+    main()
