@@ -120,7 +120,8 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 
 template <int D>
 __global__ void __launch_bounds__(kScatterBlock)
-backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t capacity, uint32_t cap_mask,
+backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int tiles_per_group, uint32_t capacity,
+                      uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
                       const float* __restrict__ grad_sliced, float* __restrict__ table_grad, BinTarget pass_bins) {
@@ -133,7 +134,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     // a time).
     const uint32_t die = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
     const uint32_t level_in_pass = j % n_pass_levels, group = (j / n_pass_levels) * kXcds + die;
-    if (static_cast<int64_t>(group) * kGroupPoints >= n_points) return;
+    const int64_t group_base = static_cast<int64_t>(group) * tiles_per_group * kScatterBlock;
+    if (group_base >= n_points) return;
     const int level = first_level + level_in_pass;
     const float w_level = window[level];
     if (w_level == 0.0f) return;
@@ -144,7 +146,6 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     const float* g1p = g0p + n_points;
     // A tile's inputs are fetched one tile ahead: their latency then overlaps the previous tile's
     // scatter instead of stalling the wave at the top of every iteration.
-    const int64_t group_base = static_cast<int64_t>(group) * kGroupPoints;
     const auto point_of = [&](int t) {  // the point this thread handles in tile t (clamped: the tail re-reads the last point)
         const int64_t n = group_base + static_cast<int64_t>(t) * kScatterBlock + threadIdx.x;
         return static_cast<int>(n < n_points ? n : n_points - 1);
@@ -153,7 +154,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     fvec<D> pos = load_point<D>(positions, nn);
     float g0 = g0p[nn], g1 = g1p[nn];
     bool streaming = false;
-    for (int t = 0; t < kScatterTiles; ++t) {
+    for (int t = 0; t < tiles_per_group; ++t) {
         const int64_t tile_base = group_base + static_cast<int64_t>(t) * kScatterBlock;
         if (tile_base >= n_points) break;
         const bool active = tile_base + threadIdx.x < n_points;
@@ -236,7 +237,8 @@ reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size
 
 template <int D, bool kTableGrad, bool kGradGrad>
 __global__ void __launch_bounds__(kScatterBlock)
-double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t capacity, uint32_t cap_mask,
+double_backward_kernel(int n_points, int n_levels, int first_level, int tiles_per_group, uint32_t capacity,
+                       uint32_t cap_mask,
                        const float* __restrict__ positions, const float* __restrict__ table,
                        const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                        const float* __restrict__ window, const float* __restrict__ double_pos_grad,
@@ -260,8 +262,8 @@ double_backward_kernel(int n_points, int n_levels, int first_level, uint32_t cap
     const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
     const float* g1p = g0p + n_points;
     bool streaming = false;
-    for (int t = 0; t < kScatterTiles; ++t) {
-        const int64_t tile_base = (static_cast<int64_t>(group) * kScatterTiles + t) * kScatterBlock;
+    for (int t = 0; t < tiles_per_group; ++t) {
+        const int64_t tile_base = (static_cast<int64_t>(group) * tiles_per_group + t) * kScatterBlock;
         if (tile_base >= n_points) break;
         if (kTableGrad && live && !streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
         const bool active = tile_base + threadIdx.x < n_points;
@@ -414,13 +416,27 @@ inline uint32_t bins_for_capacity(int capacity) {
     return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
 }
 
-inline unsigned scatter_groups(int64_t n) { return static_cast<unsigned>((n + kGroupPoints - 1) / kGroupPoints); }
+constexpr int64_t kLargeGroupsMinWorkgroups = 3000;  // about four per workgroup slot of the chip (256 CUs x 3)
+
+inline unsigned scatter_groups(int64_t n, int tiles_per_group) {
+    const int64_t group_points = static_cast<int64_t>(tiles_per_group) * kScatterBlock;
+    return static_cast<unsigned>((n + group_points - 1) / group_points);
+}
+
+// Tiles per scattering workgroup of the table backward.  Larger groups mean longer record segments
+// (less slack, longer bursts for the reducer) and fewer cache flushes; they are taken when the
+// launch still has several workgroups for every slot of the chip (measured: 3-13% faster then,
+// slower otherwise).  The double backward keeps kScatterTiles: it also gathers, a level at a time.
+inline int table_backward_tiles(int64_t n, int levels) {
+    return static_cast<int64_t>(scatter_groups(n, kScatterTilesLarge)) * levels >= kLargeGroupsMinWorkgroups ? kScatterTilesLarge
+                                                                                                            : kScatterTiles;
+}
 
 // Records one scattering workgroup may leave in one bin: its share of the group's
-// kGroupPoints*(D+1) contributions plus the flushed cache lines, with three standard deviations
+// group's contributions (D+1 per point) plus the flushed cache lines, with three standard deviations
 // of a uniform hash on top.  A segment that still overflows spills to direct atomics.
-inline uint32_t wanted_segment_capacity(int pos_dim, uint32_t n_bins) {
-    const double mean = (static_cast<double>(kGroupPoints) * (pos_dim + 1) + kCacheLines) / n_bins;
+inline uint32_t wanted_segment_capacity(int pos_dim, uint32_t n_bins, int tiles_per_group) {
+    const double mean = (static_cast<double>(tiles_per_group) * kScatterBlock * (pos_dim + 1) + kCacheLines) / n_bins;
     return static_cast<uint32_t>(mean + 3.0 * __builtin_sqrt(mean) + 8.0);
 }
 
@@ -429,17 +445,18 @@ inline size_t bin_bytes_per_level(uint32_t n_bins, uint32_t n_groups, uint32_t s
     return segments * (sizeof(uint32_t) + static_cast<size_t>(segment_capacity) * sizeof(BinRecord));
 }
 
-inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, void* workspace, size_t bytes) {
+inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int tiles_per_group, void* workspace,
+                         size_t bytes) {
     BinPlan p;
     const uint32_t n_bins = bins_for_capacity(capacity);
-    const uint32_t n_groups = scatter_groups(n);
+    const uint32_t n_groups = scatter_groups(n, tiles_per_group);
     if (workspace == nullptr || n_bins > static_cast<uint32_t>(kMaxBins)) return p;
     const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
     const size_t lost = base - reinterpret_cast<uintptr_t>(workspace);
     if (bytes < lost + 4096) return p;
     bytes -= lost + 256;
     const size_t segments = static_cast<size_t>(n_bins) * n_groups;
-    uint32_t cap = wanted_segment_capacity(pos_dim, n_bins);
+    uint32_t cap = wanted_segment_capacity(pos_dim, n_bins, tiles_per_group);
     if (bytes < bin_bytes_per_level(n_bins, n_groups, cap)) {  // not even one level at the wanted size: shrink the segments
         if (bytes < segments * (sizeof(uint32_t) + 16 * sizeof(BinRecord))) return p;
         cap = static_cast<uint32_t>((bytes / segments - sizeof(uint32_t)) / sizeof(BinRecord));
@@ -522,7 +539,13 @@ size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_le
     if (n_bins > static_cast<uint32_t>(kMaxBins)) return 0;
     if (levels_per_pass <= 0) levels_per_pass = kDefaultLevelsPerPass;
     if (levels_per_pass > nr_levels) levels_per_pass = nr_levels;
-    const size_t per_level = bin_bytes_per_level(n_bins, scatter_groups(nr_positions), wanted_segment_capacity(pos_dim, n_bins));
+    // the larger of what the two gradient calls plan for (they may group the points differently)
+    size_t per_level = 0;
+    for (const int tiles : {kScatterTiles, table_backward_tiles(nr_positions, nr_levels)}) {
+        const size_t need = bin_bytes_per_level(n_bins, scatter_groups(nr_positions, tiles),
+                                                wanted_segment_capacity(pos_dim, n_bins, tiles));
+        per_level = need > per_level ? need : per_level;
+    }
     return per_level * static_cast<size_t>(levels_per_pass) + 1024;
 }
 
@@ -578,14 +601,15 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     if (lattice_values_grad) {
         if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-        const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, workspace, workspace_bytes);
+        const int tiles_per_group = table_backward_tiles(nr_positions, nr_levels);
+        const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, tiles_per_group, workspace, workspace_bytes);
         const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
         for (int first = 0; first < nr_levels; first += per_pass) {
             const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
-            const unsigned padded_groups = (scatter_groups(nr_positions) + kXcds - 1) / kXcds * kXcds;
+            const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
             const dim3 grid(padded_groups * static_cast<unsigned>(count));
             PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD>), grid, dim3(kScatterBlock), 0, st, n,
-                                                        first, static_cast<uint32_t>(count), cap, mask, positions, scale_factor, random_shift,
+                                                        first, static_cast<uint32_t>(count), tiles_per_group, cap, mask, positions, scale_factor, random_shift,
                                                         anneal_window, grad_sliced_values, lattice_values_grad,
                                                         plan.target));
             if (int rc = check_launch()) return rc;
@@ -643,8 +667,8 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
     const dim3 block(kScatterBlock);
 #define PENC_LAUNCH_DB(TG, GG, FIRST, COUNT, TARGET)                                                             \
     PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((double_backward_kernel<DD, TG, GG>),                            \
-                                                dim3(scatter_groups(nr_positions), COUNT), block, 0, st, n, nr_levels, \
-                                                FIRST, cap, mask, positions, lattice_values, scale_factor,        \
+                                                dim3(scatter_groups(nr_positions, kScatterTiles), COUNT), block, 0, st, n, nr_levels, \
+                                                FIRST, kScatterTiles, cap, mask, positions, lattice_values, scale_factor,        \
                                                 random_shift, anneal_window, double_positions_grad,              \
                                                 grad_sliced_values, lattice_values_grad, grad_grad_sliced_values, \
                                                 TARGET))
@@ -653,7 +677,7 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
         return check_launch();
     }
     if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, workspace, workspace_bytes);
+    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, kScatterTiles, workspace, workspace_bytes);
     const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
     for (int first = 0; first < nr_levels; first += per_pass) {
         int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;

@@ -38,8 +38,8 @@ namespace penc {
 constexpr int kXcds = 8;               // accelerator dies (XCDs) of the chip; workgroup i runs on die i % kXcds
 constexpr int kBlock = 256;            // threads per workgroup of the gather-type kernels (4 wavefronts)
 constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wavefronts share one accumulate cache)
-constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks
-constexpr int kGroupPoints = kScatterBlock * kScatterTiles;
+constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks (a "group" of points) ...
+constexpr int kScatterTilesLarge = 16; // ... or this many, when the launch still has workgroups to spare
 constexpr int kCacheLinesLog2 = 11;
 constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per workgroup
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
@@ -58,7 +58,7 @@ struct BinRecord {
 };
 
 // Where the misses of the levels of one launch go.  Every scattering workgroup (a "group" of
-// kGroupPoints points at one level) owns a private segment of `segment_capacity` records in every
+// points at one level) owns a private segment of `segment_capacity` records in every
 // bin, so appending needs no global atomics and no synchronisation: the cursor is an LDS counter.
 //   records [level_in_pass][bin][group][segment_capacity]
 //   counts  [level_in_pass][bin][group]            records actually written (<= segment_capacity)
