@@ -118,7 +118,7 @@ def main():
     ap.add_argument("--no-probes", action="store_true", help="skip the memory-system probes")
     ap.add_argument("--levels-per-pass", type=int, default=0,
                     help="levels binned per scatter pass (0: library default, -1: no workspace, direct atomics)")
-    ap.add_argument("--cpu-sample", type=int, default=1 << 18, help="points in the CPU baseline sample")
+    ap.add_argument("--cpu-sample", type=int, default=1 << 20, help="points in the CPU baseline sample")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on one GPU only; --gpus N with N > 1 is not supported", file=sys.stderr)
