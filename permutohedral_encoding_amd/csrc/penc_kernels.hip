@@ -101,9 +101,14 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
         return;
     }
     const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, scale_factor + level * D);
-    const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
+    // residuals and hash steps into rank order through LDS: up to 6% faster than the select chains
+    // of vertex_hashes() / barycentric() at D = 8, equal at D = 3
+    __shared__ uint2 columns[(D + 1) * kBlock];
+    uvec<D + 1> h;
+    fvec<D + 1> sorted;
+    sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, s.delta, s.hash0, sorted, h);
+    const fvec<D + 1> w = barycentric_of_sorted<D>(sorted);
     const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
-    const fvec<D + 1> w = barycentric<D>(s.rank, s.delta);
     float acc0 = 0.0f, acc1 = 0.0f;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
@@ -188,7 +193,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
 // the position gradient itself; otherwise it is a partial buffer that reduce_level_groups_kernel
 // sums, in ascending group order, so the result is deterministic either way.  Small groups keep
 // the whole chip on the same few levels at a time (their table slices stay in L2) and give the
-// launch many more, shorter waves than one thread per point walking all levels.
+// launch many more, shorter waves than one thread per point walking all levels.  (Doing this
+// kernel's rank permutations through LDS, as the forward does, was measured: no gain.)
 template <int D>
 __global__ void __launch_bounds__(kBlock)
 backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t capacity, uint32_t cap_mask,

@@ -180,10 +180,8 @@ __device__ __forceinline__ fvec<D + 1> by_rank(ivec<D + 1> rank, fvec<D + 1> in)
     return out;
 }
 
-// Barycentric weights of the D+1 vertices (EncodingGPU.cuh:190-199).
 template <int D>
-__device__ __forceinline__ fvec<D + 1> barycentric(ivec<D + 1> rank, fvec<D + 1> delta) {
-    const fvec<D + 1> sorted = by_rank<D>(rank, delta);
+__device__ __forceinline__ fvec<D + 1> barycentric_of_sorted(fvec<D + 1> sorted) {
     fvec<D + 1> w;
     w[0] = sorted[D] + (1.0f + (0.0f - sorted[0]));
     static_for<D>(PENC_BODY(rr) {
@@ -192,6 +190,12 @@ __device__ __forceinline__ fvec<D + 1> barycentric(ivec<D + 1> rank, fvec<D + 1>
         w[r] = sorted[D - r] - sorted[D + 1 - r];
     });
     return w;
+}
+
+// Barycentric weights of the D+1 vertices (EncodingGPU.cuh:190-199).
+template <int D>
+__device__ __forceinline__ fvec<D + 1> barycentric(ivec<D + 1> rank, fvec<D + 1> delta) {
+    return barycentric_of_sorted<D>(by_rank<D>(rank, delta));
 }
 
 // Raw hashes of the D+1 vertices (EncodingGPU.cuh:212-223), by the incremental rule above.
@@ -213,19 +217,48 @@ __device__ __forceinline__ uvec<D + 1> vertex_hashes(ivec<D + 1> rank, uint32_t 
     return h;
 }
 
+// The same two results (residuals in rank order, raw vertex hashes) through LDS instead of the
+// D(D+1) compare-and-select chains above: every thread owns a column of D+1 eight-byte cells
+// (`column` points at the thread's cell of row 0, rows are `stride` cells apart, so the lanes of a
+// wave hit distinct banks), writes {delta[c], hash step of coordinate c} to row rank[c] and reads
+// the rows back in order.  A thread only reads what it wrote itself: no barrier.
+template <int D>
+__device__ __forceinline__ void sort_by_rank_lds(uint2* column, uint32_t stride, ivec<D + 1> rank, fvec<D + 1> delta,
+                                                 uint32_t hash0, fvec<D + 1>& sorted, uvec<D + 1>& hashes) {
+    static_for<D + 1>(PENC_BODY(c) {
+        PENC_INDEX(c);
+        const float d = delta[c];
+        uint2 cell;
+        cell.x = __builtin_bit_cast(uint32_t, d);
+        cell.y = hash_step<D, c>();
+        column[static_cast<uint32_t>(rank[c]) * stride] = cell;
+    });
+    uvec<D + 1> step;
+    static_for<D + 1>(PENC_BODY(m) {
+        PENC_INDEX(m);
+        const uint2 cell = column[m * stride];
+        sorted[m] = __builtin_bit_cast(float, cell.x);
+        step[m] = cell.y;
+    });
+    hashes[0] = hash0;
+    static_for<D>(PENC_BODY(r) {
+        PENC_INDEX(r);
+        hashes[r + 1] = hashes[r] + step[D - r];  // the coordinate of rank D-r starts to wrap here
+    });
+}
+
 // The three gradient chains below evaluate their sums in the same order, with the same
 // intermediate roundings, as the reference's loops, so that every term a kernel adds is the same
 // fp32 number the CPU checker computes; only the order of atomic accumulation can then differ.
 
-// d(loss)/d(barycentric) -> d(loss)/d(position) for one level (EncodingGPU.cuh:698-740).
-// dB[r] is the derivative w.r.t. the weight of vertex r.
+// d(loss)/d(barycentric) -> d(loss)/d(position) for one level (EncodingGPU.cuh:698-740), in three
+// steps.  dB[r] is the derivative w.r.t. the weight of vertex r.
+// Step 1: dE[i] = dB[D-rank[i]]/(D+1) - dB[D+1-rank[i]]/(D+1), with dB[D+1] = dB[0] (the wrap-around
+// term, :698), as a function of the rank m: diff[m] = dB[D-m]/(D+1) - dB[D+1-m]/(D+1).
 template <int D>
-__device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<D + 1> dB,
-                                                         const float* __restrict__ sf) {
+__device__ __forceinline__ fvec<D + 1> bary_grad_by_rank(fvec<D + 1> dB) {
     constexpr int D1 = D + 1;
     constexpr float kInv = 1.0f / D1;
-    // dE[i] = dB[D-rank[i]]/(D+1) - dB[D+1-rank[i]]/(D+1), with dB[D+1] = dB[0] (the wrap-around
-    // term, :698).  As a function of the rank m: diff[m] = dB[D-m]/(D+1) - dB[D+1-m]/(D+1).
     const fvec<D1> scaled = dB * kInv;
     fvec<D1> diff;
     diff[0] = scaled[D] - scaled[0];
@@ -234,8 +267,14 @@ __device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<
         constexpr int m = mm + 1;
         diff[m] = scaled[D - m] - scaled[D1 - m];
     });
-    fvec<D1> dE;
-    static_for<D1>(PENC_BODY(i) {
+    return diff;
+}
+
+// Step 2: dE[i] = diff[rank[i]], by compare-and-select chains.
+template <int D>
+__device__ __forceinline__ fvec<D + 1> pick_by_rank(ivec<D + 1> rank, fvec<D + 1> diff) {
+    fvec<D + 1> dE;
+    static_for<D + 1>(PENC_BODY(i) {
         PENC_INDEX(i);
         float acc = diff[0];
         static_for<D>(PENC_BODY(mm) {
@@ -246,7 +285,12 @@ __device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<
         });
         dE[i] = acc;
     });
-    // dP[i] = sum_{j<=i} dE[j]*sf[i] - dE[i+1]*sf[i]*(i+1)   (:729-740)
+    return dE;
+}
+
+// Step 3: dP[i] = sum_{j<=i} dE[j]*sf[i] - dE[i+1]*sf[i]*(i+1)   (:729-740)
+template <int D>
+__device__ __forceinline__ fvec<D> elevated_grad_to_pos_grad(fvec<D + 1> dE, const float* __restrict__ sf) {
     fvec<D> dP;
     static_for<D>(PENC_BODY(i) {
         PENC_INDEX(i);
@@ -259,6 +303,12 @@ __device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<
         dP[i] = acc;
     });
     return dP;
+}
+
+template <int D>
+__device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<D + 1> dB,
+                                                         const float* __restrict__ sf) {
+    return elevated_grad_to_pos_grad<D>(pick_by_rank<D>(rank, bary_grad_by_rank<D>(dB)), sf);
 }
 
 // d(loss)/d(position gradient) -> derivative w.r.t. each vertex weight (EncodingGPU.cuh:1187-1218).
