@@ -258,6 +258,19 @@ def test_full_size_adjoint_identities(name):
     assert torch.allclose(tg, tg_again, rtol=1e-3, atol=1e-6 * tg.abs().max().item())
     assert torch.equal(out, enc.forward(inp))
 
+    # every slot: the binned scatter (workspace, large point groups at this size) against the
+    # independent direct-atomics path (no workspace)
+    from permutohedral_encoding_amd import _native
+    saved = _native.LEVELS_PER_PASS
+    _native.LEVELS_PER_PASS = -1
+    try:
+        tg_direct, _ = enc.backward(inp, grad_t)
+        tg2_direct, _ = enc.double_backward_from_positions(inp, dpos_t, grad_t)
+    finally:
+        _native.LEVELS_PER_PASS = saved
+    assert torch.allclose(tg, tg_direct, rtol=1e-3, atol=1e-5 * tg.abs().max().item())
+    assert torch.allclose(tg2, tg2_direct, rtol=1e-3, atol=1e-5 * tg2.abs().max().item())
+
 
 def test_full_size_constant_table_gives_window():
     w = wl.WORKLOADS["c2"]
