@@ -231,7 +231,10 @@ __device__ __forceinline__ void sort_by_rank_lds(uint2* column, uint32_t stride,
         uint2 cell;
         cell.x = __builtin_bit_cast(uint32_t, d);
         cell.y = hash_step<D, c>();
-        column[static_cast<uint32_t>(rank[c]) * stride] = cell;
+        // ranks of finite points are a permutation of 0..D; the clamp keeps a point with NaN or
+        // overflowing coordinates inside its own column
+        const int row = rank[c] < 0 ? 0 : (rank[c] > D ? D : rank[c]);
+        column[static_cast<uint32_t>(row) * stride] = cell;
     });
     uvec<D + 1> step;
     static_for<D + 1>(PENC_BODY(m) {

@@ -369,3 +369,34 @@ def test_position_gradient_with_and_without_workspace():
         assert np.all(np.abs(got - want) <= SUM_RTOL * (np.abs(want) + scale))
         results.append(got)
     assert np.array_equal(results[0], results[2])
+
+
+def test_non_finite_points_do_not_disturb_their_neighbours():
+    """A point with NaN, infinite or overflowing coordinates gets garbage (as in the reference), but
+    the other points of its workgroup must come out exactly as without it, and nothing may fault."""
+    d, cap, n = 3, 1 << 14, 4096
+    p = random_problem(d, n, 8, cap, seed=31, sigma_range=(1.0, 1e-3))
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    clean = gpu_input(p)
+    grad, dpos = to_gpu(p["grad"]), to_gpu(p["dpos"])
+    out_clean = enc.forward(clean)
+    _, pg_clean = enc.backward(clean, grad)
+    _, ggs_clean = enc.double_backward_from_positions(clean, dpos, grad)
+
+    bad_rows = [5, 64, 65, 1000, 4095]
+    dirty_pos = p["pos"].copy()
+    for row, value in zip(bad_rows, [np.nan, np.inf, -np.inf, 3e38, -1e30]):
+        dirty_pos[row, row % d] = value
+    q = dict(p)
+    q["pos"] = dirty_pos
+    dirty = gpu_input(q)
+    out = enc.forward(dirty)
+    tg, pg = enc.backward(dirty, grad)
+    tg2, ggs = enc.double_backward_from_positions(dirty, dpos, grad)
+    torch.cuda.synchronize()
+    keep = torch.ones(n, dtype=torch.bool, device="cuda")
+    keep[bad_rows] = False
+    assert torch.equal(out[:, :, keep], out_clean[:, :, keep])
+    assert torch.equal(pg[keep], pg_clean[keep])
+    assert torch.equal(ggs[:, :, keep], ggs_clean[:, :, keep])
+    assert tg.shape == tg2.shape == (8, cap, 2)
