@@ -97,6 +97,16 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* The table gradient of penc_backward, reading the upstream gradient as the layer after the encoding
+ * produces it: rows grad_rows[n][2*level + feature] of grad_row_stride floats (even, >= 2*nr_levels;
+ * 8-byte aligned), instead of [level][feature][n].  lattice_values_grad is cleared first.
+ * Replaces: the strided `.contiguous()` copy of src/pytorch_modules/funcs.py:47 followed by
+ * Encoding<D,2>::backward with only require_lattice_values_grad set (src/Encoding.cu:112-215). */
+int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                 const float* positions, const float* scale_factor, const float* random_shift,
+                                 const float* anneal_window, const float* grad_rows, int64_t grad_row_stride,
+                                 float* lattice_values_grad, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Double backward from d(loss)/d(positions_grad): gradient w.r.t. lattice_values and w.r.t.
  * grad_sliced_values ([L+E][2][N], zeros in the extra levels).  Either output may be NULL.
  * lattice_values_grad is cleared by the library first.

@@ -31,6 +31,9 @@ _SIGNATURES = {
     "penc_backward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                      _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                      ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_backward_table_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                    _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
+                                                    ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_double_backward_from_positions": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
                                                            ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int,
@@ -120,6 +123,17 @@ def _check_f32_gpu(t, name, ndim):
     _require(t.is_cuda, f"{name} should be in GPU memory. Please call .cuda() on the tensor")
     _require(t.dtype == torch.float32, f"{name} should be of type float")
     _require(t.dim() == ndim, f"{name} should have {ndim} dimensions, however it has sizes {tuple(t.shape)}")
+
+
+def is_row_major_view(grad):
+    """True for a (L, 2, N) *view* of rows grad_rows[n][2*level + feature] (the upstream gradient of the
+    module's (N, 2L) output seen through its permute+reshape): the table gradient can read that as it is."""
+    if grad.dim() != 3 or not grad.is_cuda or grad.dtype != torch.float32 or grad.is_contiguous():
+        return False
+    levels, feat, n = grad.shape
+    s_level, s_feat, s_point = grad.stride()
+    return (feat == 2 and n > 0 and s_level == 2 and s_feat == 1 and s_point >= 2 * levels and s_point % 2 == 0
+            and grad.data_ptr() % 8 == 0 and s_point * n < 2 ** 31)
 
 
 def level_major_gradient(grad):
@@ -217,9 +231,10 @@ class EncodingWrapper:
             fp.m_scale_factor = fp.m_scale_factor.to(dev)
         return pos.contiguous(), lv, shift.contiguous(), win.contiguous(), levels, lv.shape[1]
 
-    def _check_grad(self, grad, levels, extra, n):
+    def _check_grad(self, grad, levels, extra, n, allow_rows=False):
         _check_f32_gpu(grad, "grad_sliced_values_monolithic", 3)
-        _require(grad.is_contiguous(), "Grad sliced values needs to be contiguous. Please call .contiguous() on it")
+        _require(grad.is_contiguous() or (allow_rows and is_row_major_view(grad)),
+                 "Grad sliced values needs to be contiguous. Please call .contiguous() on it")
         _require(grad.shape == (levels + extra, self.nr_feat, n),
                  "grad_sliced_values_monolithic should be nr_resolutions x val_dim x nr_positions")
 
@@ -243,13 +258,20 @@ class EncodingWrapper:
         pos, lv, shift, win, levels, cap = self._check_common(inp)
         n = pos.shape[0]
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
-        self._check_grad(grad_sliced_values_monolithic, levels, extra, n)
+        table_only = inp.m_require_lattice_values_grad and not inp.m_require_positions_grad
+        self._check_grad(grad_sliced_values_monolithic, levels, extra, n, allow_rows=table_only)
         lv_grad = torch.empty_like(lv) if inp.m_require_lattice_values_grad else None
         pos_grad = torch.empty_like(pos) if inp.m_require_positions_grad else None
         if lv_grad is None and pos_grad is None:
             return None, None
         with torch.cuda.device(pos.device):
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None)
+            if not grad_sliced_values_monolithic.is_contiguous():  # rows (N, 2(L+E)): read in place, no copy
+                _check(lib().penc_backward_table_rowmajor(
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
+                    _ptr(grad_sliced_values_monolithic), grad_sliced_values_monolithic.stride(2), _ptr(lv_grad),
+                    _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
+                return lv_grad, None
             _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
                                        _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
                                        _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(pos_grad),

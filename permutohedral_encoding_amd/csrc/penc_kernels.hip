@@ -123,13 +123,18 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 // ------------------------------------------------------------------------------------------
 // backward w.r.t. the table (EncodingGPU.cuh:259-414)
 
-template <int D>
+// kRowMajor: the upstream gradient is read as rows grad[n][2*level + feature] of `grad_row_stride`
+// floats (what the layer after the encoding produces) instead of [level][feature][n].  A die walks
+// all levels of a group of points back to back, so the rows are fetched from memory about once
+// although every level only uses 8 bytes of each.
+template <int D, bool kRowMajor>
 __global__ void __launch_bounds__(kScatterBlock)
 backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int tiles_per_group, uint32_t capacity,
                       uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
-                      const float* __restrict__ grad_sliced, float* __restrict__ table_grad, BinTarget pass_bins) {
+                      const float* __restrict__ grad_sliced, int64_t grad_row_stride, float* __restrict__ table_grad,
+                      BinTarget pass_bins) {
     __shared__ ScatterState state;
     // Workgroups are dealt round-robin to the kXcds dies, each with an L2 of its own.  The j-th
     // workgroup of a die takes level j % levels of one group of points: a die works through all
@@ -147,8 +152,17 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
     scatter_begin(state);
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
-    const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
-    const float* g1p = g0p + n_points;
+    const auto load_grad = [&](int n, float& g0, float& g1) {
+        if constexpr (kRowMajor) {
+            const float2 g = *reinterpret_cast<const float2*>(grad_sliced + static_cast<int64_t>(n) * grad_row_stride + 2 * level);
+            g0 = g.x;
+            g1 = g.y;
+        } else {
+            const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
+            g0 = g0p[n];
+            g1 = g0p[static_cast<size_t>(n_points) + n];
+        }
+    };
     // A tile's inputs are fetched one tile ahead: their latency then overlaps the previous tile's
     // scatter instead of stalling the wave at the top of every iteration.
     const auto point_of = [&](int t) {  // the point this thread handles in tile t (clamped: the tail re-reads the last point)
@@ -157,7 +171,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
     };
     int nn = point_of(0);
     fvec<D> pos = load_point<D>(positions, nn);
-    float g0 = g0p[nn], g1 = g1p[nn];
+    float g0, g1;
+    load_grad(nn, g0, g1);
     bool streaming = false;
     for (int t = 0; t < tiles_per_group; ++t) {
         const int64_t tile_base = group_base + static_cast<int64_t>(t) * kScatterBlock;
@@ -165,7 +180,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
         const bool active = tile_base + threadIdx.x < n_points;
         const int nn_next = point_of(t + 1);
         const fvec<D> pos_next = load_point<D>(positions, nn_next);
-        const float g0_next = g0p[nn_next], g1_next = g1p[nn_next];
+        float g0_next, g1_next;
+        load_grad(nn_next, g0_next, g1_next);
         if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
@@ -519,6 +535,41 @@ inline unsigned tiles(int64_t n) { return static_cast<unsigned>((n + kBlock - 1)
 
 using namespace penc;
 
+// The table gradient of penc_backward / penc_backward_table_rowmajor: clear, scatter, reduce the
+// bins, in as many passes over the levels as the workspace asks for.  grad_row_stride == 0 means
+// the [level][feature][n] layout, otherwise the gradient is rows of that many floats.
+static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
+                          const float* scale_factor, const float* random_shift, const float* anneal_window,
+                          const float* grad, int64_t grad_row_stride, float* lattice_values_grad, void* workspace,
+                          size_t workspace_bytes, hipStream_t st) {
+    const int n = static_cast<int>(nr_positions);
+    const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
+    if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
+    const int tiles_per_group = table_backward_tiles(nr_positions, nr_levels);
+    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, tiles_per_group, workspace, workspace_bytes);
+    const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
+    for (int first = 0; first < nr_levels; first += per_pass) {
+        const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
+        const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
+        const dim3 grid(padded_groups * static_cast<unsigned>(count));
+#define PENC_LAUNCH_TABLE(ROW_MAJOR)                                                                                       \
+    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR>), grid, dim3(kScatterBlock), 0, st, n, \
+                                                first, static_cast<uint32_t>(count), tiles_per_group, cap, mask, positions,  \
+                                                scale_factor, random_shift, anneal_window, grad, grad_row_stride,            \
+                                                lattice_values_grad, plan.target))
+        if (grad_row_stride != 0) {
+            PENC_LAUNCH_TABLE(true);
+        } else {
+            PENC_LAUNCH_TABLE(false);
+        }
+#undef PENC_LAUNCH_TABLE
+        if (int rc = check_launch()) return rc;
+        if (plan.enabled)
+            if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, lattice_values_grad, st)) return rc;
+    }
+    return PENC_OK;
+}
+
 extern "C" {
 
 const char* penc_status_string(int status) {
@@ -605,24 +656,10 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
-    if (lattice_values_grad) {
-        if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-        const int tiles_per_group = table_backward_tiles(nr_positions, nr_levels);
-        const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, tiles_per_group, workspace, workspace_bytes);
-        const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
-        for (int first = 0; first < nr_levels; first += per_pass) {
-            const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
-            const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
-            const dim3 grid(padded_groups * static_cast<unsigned>(count));
-            PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD>), grid, dim3(kScatterBlock), 0, st, n,
-                                                        first, static_cast<uint32_t>(count), tiles_per_group, cap, mask, positions, scale_factor, random_shift,
-                                                        anneal_window, grad_sliced_values, lattice_values_grad,
-                                                        plan.target));
-            if (int rc = check_launch()) return rc;
-            if (plan.enabled)
-                if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, lattice_values_grad, st)) return rc;
-        }
-    }
+    if (lattice_values_grad)
+        if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+                                    anneal_window, grad_sliced_values, 0, lattice_values_grad, workspace, workspace_bytes, st))
+            return rc;
     if (positions_grad) {
         // levels in groups of kPosLevelsPerGroup when the workspace can hold the partial sums
         // (the table-gradient scatter above is done with it: same stream), else one group
@@ -650,6 +687,22 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
         }
     }
     return PENC_OK;
+}
+
+int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                 const float* positions, const float* scale_factor, const float* random_shift,
+                                 const float* anneal_window, const float* grad_rows, int64_t grad_row_stride,
+                                 float* lattice_values_grad, void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
+    if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_rows || !lattice_values_grad)
+        return PENC_ERR_NULL_POINTER;
+    if (grad_row_stride < 2 * static_cast<int64_t>(nr_levels) || (grad_row_stride & 1) != 0 ||
+        grad_row_stride * nr_positions >= (int64_t{1} << 31))
+        return PENC_ERR_BAD_SIZE;
+    if (!aligned8(lattice_values_grad) || !aligned8(grad_rows)) return PENC_ERR_MISALIGNED;
+    return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
+                          grad_rows, grad_row_stride, lattice_values_grad, workspace, workspace_bytes,
+                          static_cast<hipStream_t>(stream));
 }
 
 int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,

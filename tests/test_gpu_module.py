@@ -203,3 +203,68 @@ def test_level_major_gradient_paths():
     assert torch.equal(_native.level_major_gradient(odd), odd.contiguous())
     c = torch.randn(6, 2, 100, device="cuda")
     assert _native.level_major_gradient(c) is c
+
+
+@pytest.mark.parametrize("d,n,levels,cap,concat", [(3, 20000, 8, 1 << 14, False), (4, 5001, 6, 50000, True), (2, 70000, 24, 1 << 15, False)])
+def test_table_gradient_from_row_major_upstream_gradient(d, n, levels, cap, concat):
+    """The table gradient read straight from rows grad[n][2*level+feature] must equal the oracle's on
+    the level-major copy (same terms, same tolerance as any atomic sum), also with the extra
+    columns of concatenated points and a padded row stride."""
+    from permutohedral_encoding_amd import _native
+    from helpers import random_problem, make_encoding, gpu_input, assert_sum_close
+    SUM_RTOL = 1e-4  # atomically accumulated gradients, relative to the sum of magnitudes of their terms
+    from oracle import api as orc
+    p = random_problem(d, n, levels, cap, seed=41, sigma_range=(1.0, 1e-3))
+    enc, fp = make_encoding(d, p["sigmas"], p["shift"], concat_points=concat)
+    extra = _native.extra_levels(d, 2, concat)
+    cols = 2 * (levels + extra)
+    rng = np.random.default_rng(5)
+    rows = torch.from_numpy(rng.standard_normal((n, cols + 2)).astype(np.float32)).cuda()   # padded rows
+    view = rows[:, :cols].reshape(n, levels + extra, 2).permute(1, 2, 0)
+    assert _native.is_row_major_view(view)
+    inp = gpu_input(p, need_pos_grad=False)   # table gradient only
+    tg, pg = enc.backward(inp, view)
+    assert pg is None
+    sf = orc.scale_factors(d, p["sigmas"])
+    level_major = np.ascontiguousarray(view[:levels].cpu().numpy())
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], level_major, cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient from rows")
+    tg_copy, _ = enc.backward(inp, view.contiguous())
+    assert torch.allclose(tg, tg_copy, rtol=1e-3, atol=1e-6 * tg_copy.abs().max().item())
+
+
+def test_row_major_entry_point_rejects_bad_strides():
+    from permutohedral_encoding_amd import _native
+    lib = _native.lib()
+    t = torch.zeros(64, device="cuda")
+    args = lambda stride, grad: (3, 2, 4, 2, 8, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), grad, stride,
+                                 t.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+    assert lib.penc_backward_table_rowmajor(*args(3, t.data_ptr())) == 2      # stride < 2 * levels
+    assert lib.penc_backward_table_rowmajor(*args(5, t.data_ptr())) == 2      # odd stride
+    assert lib.penc_backward_table_rowmajor(*args(4, t.data_ptr() + 4)) == 5  # rows not 8-byte aligned
+    assert lib.penc_backward_table_rowmajor(*args(4, None)) == 1
+
+
+def test_module_backward_reads_the_upstream_gradient_in_place():
+    """Table-only training takes no layout copy at all; with position gradients the copy is made."""
+    import permutohedral_encoding_amd as pe
+    from permutohedral_encoding_amd import _native
+    torch.manual_seed(3)
+    enc = pe.PermutoEncoding(3, 1 << 14, 8, 2, np.geomspace(1.0, 1e-3, 8))
+    pts = torch.rand(5000, 3, device="cuda")
+    up = torch.randn(5000, 16, device="cuda")  # a row-major upstream gradient, as a consumer that copies would send
+    calls = []
+    real = _native.level_major_gradient
+    _native_funcs = __import__("permutohedral_encoding_amd.funcs", fromlist=["x"])
+    _native_funcs.level_major_gradient = lambda g: (calls.append(1), real(g))[1]
+    try:
+        enc(pts).backward(up)
+        g_table_only = enc.lattice_values.grad.clone()
+        assert calls == []
+        enc.lattice_values.grad = None
+        pts_g = pts.clone().requires_grad_(True)
+        enc(pts_g).backward(up)
+        assert calls == [1]
+    finally:
+        _native_funcs.level_major_gradient = real
+    assert torch.allclose(g_table_only, enc.lattice_values.grad, rtol=1e-3, atol=1e-6 * g_table_only.abs().max().item())
