@@ -438,6 +438,7 @@ inline uint32_t bins_for_capacity(int capacity) {
     return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
 }
 
+constexpr int64_t kMinSlotsPerContribution = 8;
 constexpr int64_t kLargeGroupsMinWorkgroups = 3000;  // about four per workgroup slot of the chip (256 CUs x 3)
 
 inline unsigned scatter_groups(int64_t n, int tiles_per_group) {
@@ -473,6 +474,9 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int t
     const uint32_t n_bins = bins_for_capacity(capacity);
     const uint32_t n_groups = scatter_groups(n, tiles_per_group);
     if (workspace == nullptr || n_bins > static_cast<uint32_t>(kMaxBins)) return p;
+    // few contributions per slot: the reducer's fixed cost per bin (clearing and flushing 128 KiB of
+    // LDS) exceeds what direct atomics cost (measured crossover: one contribution per eight slots)
+    if (n * (pos_dim + 1) * kMinSlotsPerContribution <= capacity) return p;
     const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
     const size_t lost = base - reinterpret_cast<uintptr_t>(workspace);
     if (bytes < lost + 4096) return p;

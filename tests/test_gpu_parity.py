@@ -400,3 +400,18 @@ def test_non_finite_points_do_not_disturb_their_neighbours():
     assert torch.equal(pg[keep], pg_clean[keep])
     assert torch.equal(ggs[:, :, keep], ggs_clean[:, :, keep])
     assert tg.shape == tg2.shape == (8, cap, 2)
+
+
+def test_many_bins_and_few_contributions_per_slot():
+    """A 2^22-slot table: with enough points the scatter bins into 512 slot ranges (the records are
+    appended one by one, not sorted by wave), with few points it goes straight to atomics (less than
+    one contribution per eight slots).  Both against the oracle."""
+    d, cap, levels = 3, 1 << 22, 3
+    for n in (140000, 3000):
+        p = random_problem(d, n, levels, cap, seed=12, sigma_range=(3e-2, 1e-3))
+        sf = orc.scale_factors(d, p["sigmas"])
+        enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+        inp = gpu_input(p, need_pos_grad=False)
+        tg, _ = enc.backward(inp, to_gpu(p["grad"]))
+        want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+        assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, {n} points")
