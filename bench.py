@@ -70,6 +70,43 @@ def cpu_baseline(w, inputs, sample_points, reps=5):
     }
 
 
+def module_level(torch, w, inputs, steps, warmup):
+    """The same step through the PyTorch module and autograd, as a user of the package pays it: output
+    allocation, the (N, 2L) view, a row-major upstream gradient of shape (N, 2L) and, if the workload
+    has them, position gradients.  Not part of `value`."""
+    import permutohedral_encoding_amd as pe
+    enc = pe.PermutoEncoding(w.pos_dim, w.capacity, w.nr_levels, 2, inputs["sigmas"])
+    with torch.no_grad():
+        enc.lattice_values.copy_(torch.from_numpy(inputs["table"]))
+        enc.random_shift_per_level.copy_(torch.from_numpy(inputs["shift"]))
+    pos = torch.from_numpy(inputs["pos"]).cuda()
+    if "backward_pos" in w.phases:
+        pos.requires_grad_(True)
+    window = torch.from_numpy(inputs["window"]).cuda()
+    upstream = torch.from_numpy(np.ascontiguousarray(inputs["grad"].transpose(2, 0, 1).reshape(w.nr_points, -1))).cuda()
+    backward = any(p.startswith("backward") for p in w.phases)
+
+    def step():
+        if backward:
+            enc(pos, window).backward(upstream)
+            enc.lattice_values.grad = None
+            pos.grad = None
+        else:
+            with torch.no_grad():
+                enc(pos, window)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    return {"ms_per_step": ms, "point_levels_per_s": w.point_levels / (ms * 1e-3),
+            "what": "PermutoEncoding forward" + (" + autograd backward from a row-major (N, 2L) upstream gradient" if backward else "")}
+
+
 def run_probes(torch, native, capacity, n_threads, per_thread):
     """Streaming copy, random 8-byte gathers and random fp32 atomic pairs over one level-sized slice."""
     lib = native.lib()
@@ -116,6 +153,7 @@ def main():
     ap.add_argument("--workload", default="c2")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-probes", action="store_true", help="skip the memory-system probes")
+    ap.add_argument("--no-module", action="store_true", help="skip the module-level (autograd) timing")
     ap.add_argument("--levels-per-pass", type=int, default=0,
                     help="levels binned per scatter pass (0: library default, -1: no workspace, direct atomics)")
     ap.add_argument("--cpu-sample", type=int, default=1 << 20, help="points in the CPU baseline sample")
@@ -199,9 +237,12 @@ def main():
     elapsed = time.perf_counter() - t0
 
     ms_per_step = elapsed / args.steps * 1e3
-    phase_ms = {}
+    phase_ms, phase_median, phase_min = {}, {}, {}
     for j, (name, _) in enumerate(phases):
-        phase_ms[name] = float(np.mean([events[k][j].elapsed_time(events[k][j + 1]) for k in range(args.steps)]))
+        samples = [events[k][j].elapsed_time(events[k][j + 1]) for k in range(args.steps)]
+        phase_ms[name] = float(np.mean(samples))
+        phase_median[name] = float(np.median(samples))
+        phase_min[name] = float(np.min(samples))
 
     ab = algorithmic_bytes(w)
     phase_bytes = {"forward": ab["forward"]}
@@ -239,6 +280,8 @@ def main():
         "config": {"workload": f"{w.name}: pos_dim={d} levels={levels} capacity=2^{cap.bit_length() - 1} feat=2 "
                                f"points=2^{n.bit_length() - 1} phases={'+'.join(p for p, _ in phases)}"},
         "phases_ms": phase_ms,
+        "phases_ms_median": phase_median,
+        "phases_ms_min": phase_min,
         "phases_point_levels_per_s": {k: w.point_levels / (v * 1e-3) for k, v in phase_ms.items()},
         "phases_algorithmic_GBps": {k: phase_bytes[k] * w.point_levels / (v * 1e-3) / 1e9 for k, v in phase_ms.items()},
         "roofline": roofline,
@@ -270,6 +313,8 @@ def main():
                 "note": "measured HBM bytes per launch / measured phase time; the forward is bound by random 8-byte "
                         "gathers (see probes.gather_Gacc_per_s), the table backward by streaming its slot-range records",
             }
+    if not args.no_module:
+        result["module_level"] = module_level(torch, w, inputs, args.steps, args.warmup)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(w, inputs, args.cpu_sample)
     print(json.dumps(result))
