@@ -304,18 +304,19 @@ double_backward_kernel(int n_points, int n_levels, int first_level, int tiles_pe
             if constexpr (kGradGrad) v = load_vertices<D>(level_table, h, capacity, cap_mask);
             // dB[r] * w_level, then times g_f or times the vertex value (:1244-1245, :1484-1485)
             const fvec<D + 1> wr = pos_grad_grad_to_bary<D>(s.rank, load_point<D>(double_pos_grad, nn), sf) * w_level;
+            // the scatter does not need the gathered table entries: it runs while they are in flight
+            if constexpr (kTableGrad) {
+                const float g0 = g0p[nn], g1 = g1p[nn];
+                const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
+                                                      streaming, slot, wr * g0, wr * g1);
+                if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
+            }
             if constexpr (kGradGrad) {
                 static_for<D + 1>(PENC_BODY(r) {
                     PENC_INDEX(r);
                     gg0 += wr[r] * v.f0[r];
                     gg1 += wr[r] * v.f1[r];
                 });
-            }
-            if constexpr (kTableGrad) {
-                const float g0 = g0p[nn], g1 = g1p[nn];
-                const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
-                                                      streaming, slot, wr * g0, wr * g1);
-                if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
             }
         }
         if (kGradGrad && active) {
