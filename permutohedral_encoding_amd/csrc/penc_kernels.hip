@@ -254,22 +254,28 @@ reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size
 }
 
 // ------------------------------------------------------------------------------------------
-// double backward from d(loss)/d(position gradient): both halves in one pass
+// double backward from d(loss)/d(position gradient): either half, or both in one pass
 // (EncodingGPU.cuh:1016-1257 scatter into the table gradient, 1260-1493 grad of grad_sliced)
 
 template <int D, bool kTableGrad, bool kGradGrad>
 __global__ void __launch_bounds__(kScatterBlock)
-double_backward_kernel(int n_points, int n_levels, int first_level, int tiles_per_group, uint32_t capacity,
-                       uint32_t cap_mask,
+double_backward_kernel(int n_points, int n_levels, int first_level, int tiles_per_group, uint32_t interleaved_levels,
+                       uint32_t capacity, uint32_t cap_mask,
                        const float* __restrict__ positions, const float* __restrict__ table,
                        const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                        const float* __restrict__ window, const float* __restrict__ double_pos_grad,
                        const float* __restrict__ grad_sliced, float* __restrict__ table_grad,
                        float* __restrict__ grad_grad_sliced, BinTarget pass_bins) {
     __shared__ ScatterState state;
-    // a level at a time (blockIdx.y), unlike backward_table_kernel: this kernel gathers from the
-    // table, and interleaving levels was measured equal to 13% slower (the slices fall out of L2)
-    const uint32_t level_in_pass = blockIdx.y, group = blockIdx.x;
+    // a level at a time (blockIdx.y) whenever the kernel gathers from the table: interleaving levels
+    // was then measured equal to 13% slower (the slices fall out of L2)
+    uint32_t level_in_pass = blockIdx.y, group = blockIdx.x;
+    if (interleaved_levels != 0u) {  // the table-gradient half on its own: dealt to the dies like backward_table_kernel
+        const uint32_t die = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
+        level_in_pass = j % interleaved_levels;
+        group = (j / interleaved_levels) * kXcds + die;
+        if (static_cast<int64_t>(group) * tiles_per_group * kScatterBlock >= n_points) return;
+    }
     const int level = first_level + level_in_pass;
     const bool extra_level = level >= n_levels;  // concat levels: zeros (:1290-1295)
     const float w_level = extra_level ? 0.0f : window[level];
@@ -439,6 +445,7 @@ inline uint32_t bins_for_capacity(int capacity) {
     return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
 }
 
+constexpr int kSplitDoubleBackwardMaxDim = 4;
 constexpr int64_t kMinSlotsPerContribution = 8;
 constexpr int64_t kLargeGroupsMinWorkgroups = 3000;  // about four per workgroup slot of the chip (256 CUs x 3)
 
@@ -729,28 +736,36 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     const dim3 block(kScatterBlock);
-#define PENC_LAUNCH_DB(TG, GG, FIRST, COUNT, TARGET)                                                             \
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((double_backward_kernel<DD, TG, GG>),                            \
-                                                dim3(scatter_groups(nr_positions, kScatterTiles), COUNT), block, 0, st, n, nr_levels, \
-                                                FIRST, kScatterTiles, cap, mask, positions, lattice_values, scale_factor,        \
-                                                random_shift, anneal_window, double_positions_grad,              \
-                                                grad_sliced_values, lattice_values_grad, grad_grad_sliced_values, \
-                                                TARGET))
-    if (!lattice_values_grad) {
-        PENC_LAUNCH_DB(false, true, 0, nr_levels + extra, BinTarget{});
-        return check_launch();
+#define PENC_LAUNCH_DB(TG, GG, GRID, FIRST, TILES, INTERLEAVED, TARGET)                                               \
+    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((double_backward_kernel<DD, TG, GG>), GRID, block, 0, st, n, nr_levels,  \
+                                                FIRST, TILES, INTERLEAVED, cap, mask, positions, lattice_values,         \
+                                                scale_factor, random_shift, anneal_window, double_positions_grad,       \
+                                                grad_sliced_values, lattice_values_grad, grad_grad_sliced_values, TARGET))
+    // Both halves in one kernel share the simplex search, but the table-gradient half on its own can
+    // interleave levels and take large groups like backward_table_kernel.  Measured: two kernels are
+    // 2-9% faster up to D = 4 and 13% slower at D = 8, where the search is the expensive part.
+    const bool split = lattice_values_grad && grad_grad_sliced_values && pos_dim <= kSplitDoubleBackwardMaxDim;
+    const unsigned groups8 = scatter_groups(nr_positions, kScatterTiles);
+    if (grad_grad_sliced_values && (!lattice_values_grad || split)) {
+        PENC_LAUNCH_DB(false, true, dim3(groups8, nr_levels + extra), 0, kScatterTiles, 0u, BinTarget{});
+        if (int rc = check_launch()) return rc;
+        if (!lattice_values_grad) return PENC_OK;
     }
+    const bool alone = !grad_grad_sliced_values || split;  // the table-gradient half runs without the gathers
+    const int tiles_per_group = alone ? table_backward_tiles(nr_positions, nr_levels) : kScatterTiles;
     if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, kScatterTiles, workspace, workspace_bytes);
+    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, tiles_per_group, workspace, workspace_bytes);
     const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
     for (int first = 0; first < nr_levels; first += per_pass) {
         int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
         const int scatter_levels = count;
-        if (first + count == nr_levels && grad_grad_sliced_values) count += extra;  // the zero-filled concat levels
-        if (grad_grad_sliced_values) {
-            PENC_LAUNCH_DB(true, true, first, count, plan.target);
+        if (alone) {
+            const unsigned padded = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
+            PENC_LAUNCH_DB(true, false, dim3(padded * static_cast<unsigned>(count)), first, tiles_per_group,
+                           static_cast<uint32_t>(count), plan.target);
         } else {
-            PENC_LAUNCH_DB(true, false, first, count, plan.target);
+            if (first + count == nr_levels) count += extra;  // the zero-filled concat levels
+            PENC_LAUNCH_DB(true, true, dim3(groups8, count), first, kScatterTiles, 0u, plan.target);
         }
         if (int rc = check_launch()) return rc;
         if (plan.enabled)
