@@ -251,7 +251,7 @@ def main():
     kernel_names = {"forward": "forward_kernel",
                     "backward": "+".join((["fill_zero_kernel", "backward_table_kernel", "bin_reduce_kernel"] if want_table else [])
                                          + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else [])),
-                    "double_backward": "fill_zero_kernel+double_backward_kernel+bin_reduce_kernel"}
+                    "double_backward": "grad_grad_kernel+fill_zero_kernel+backward_table_kernel<second order>+bin_reduce_kernel"}
     dominant = max(phase_ms, key=phase_ms.get)
     achieved = phase_bytes[dominant] * w.point_levels / (phase_ms[dominant] * 1e-3) / 1e9
     traffic = None

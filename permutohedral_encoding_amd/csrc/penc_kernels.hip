@@ -1,22 +1,19 @@
 // HIP kernels (gfx950, wave64) and C-ABI entry points of the permutohedral-lattice hash encoding.
 //
-// Work decomposition
-//   forward, table backward, double backward : one thread per (point, level); blockIdx.y is the
-//       level, so consecutive workgroups work on the same 8*capacity-byte slice of the table and
-//       the level's scale factors / shifts / window weight are wave-uniform (scalar loads).
-//   position backward : one thread per point, looping over the levels and summing in registers,
-//       so the result is written once, without atomics and in a fixed order (the reference needs
-//       D atomics per point-level because it gives each level its own block,
+// Work decomposition (one thread per (point, level) everywhere)
+//   forward, grad-of-grad (the gathering half of the double backward) : blockIdx.y is the level, so
+//       consecutive workgroups work on the same 8*capacity-byte slice of the table, which stays in
+//       L2, and the level's scale factors / shifts / window weight are wave-uniform (scalar loads).
+//   position backward : a thread sums a group of two levels in registers; the per-group partial
+//       sums are reduced in a fixed order, without atomics (the reference needs D atomics per
+//       point-level because it gives each level its own block,
 //       kernels/permutohedral_encoding/EncodingGPU.cuh:745-750).
+//   table backward (first order and the scattering half of the double backward) : workgroups of
+//       512 threads walk groups of 8 or 16 tiles of points; neighbouring workgroups of a die take
+//       the same points at different levels.  The scatter itself (LDS accumulate cache, slot-range
+//       bins, direct atomics) is described in penc_scatter.hpp.
 //   A level whose anneal-window weight is exactly 0 contributes exactly 0 everywhere (for finite
 //   table values), so such levels skip the table traffic and only store their zeros.
-//
-// Table gradient.  Thousands of points share a handful of lattice vertices at the coarse levels,
-// so the scatter-add goes through two stages of combining before it reaches global fp32 atomics:
-// a wave whose lanes all hit the same slot reduces with DPP and issues one atomic, and every
-// workgroup accumulates into a small direct-mapped cache in LDS (tag = slot) that is flushed once
-// at the end; a slot that loses its LDS line to another slot falls through to a global atomic, so
-// the result does not depend on the cache ever hitting.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -127,14 +124,17 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 // floats (what the layer after the encoding produces) instead of [level][feature][n].  A die walks
 // all levels of a group of points back to back, so the rows are fetched from memory about once
 // although every level only uses 8 bytes of each.
-template <int D, bool kRowMajor>
+// kSecondOrder: the table-gradient half of the double backward (EncodingGPU.cuh:1016-1257): the
+// vertex weights are the derivatives of the barycentric weights along `double_pos_grad` instead of
+// the barycentric weights themselves; everything else is the same scatter.
+template <int D, bool kRowMajor, bool kSecondOrder>
 __global__ void __launch_bounds__(kScatterBlock)
 backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int tiles_per_group, uint32_t capacity,
                       uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
-                      const float* __restrict__ grad_sliced, int64_t grad_row_stride, float* __restrict__ table_grad,
-                      BinTarget pass_bins) {
+                      const float* __restrict__ grad_sliced, int64_t grad_row_stride,
+                      const float* __restrict__ double_pos_grad, float* __restrict__ table_grad, BinTarget pass_bins) {
     __shared__ ScatterState state;
     // Workgroups are dealt round-robin to the kXcds dies, each with an L2 of its own.  The j-th
     // workgroup of a die takes level j % levels of one group of points: a die works through all
@@ -171,6 +171,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
     };
     int nn = point_of(0);
     fvec<D> pos = load_point<D>(positions, nn);
+    fvec<D> q = 0.0f;
+    if constexpr (kSecondOrder) q = load_point<D>(double_pos_grad, nn);
     float g0, g1;
     load_grad(nn, g0, g1);
     bool streaming = false;
@@ -180,12 +182,19 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
         const bool active = tile_base + threadIdx.x < n_points;
         const int nn_next = point_of(t + 1);
         const fvec<D> pos_next = load_point<D>(positions, nn_next);
+        fvec<D> q_next = 0.0f;
+        if constexpr (kSecondOrder) q_next = load_point<D>(double_pos_grad, nn_next);
         float g0_next, g1_next;
         load_grad(nn_next, g0_next, g1_next);
         if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
-        const fvec<D + 1> w = barycentric<D>(s.rank, s.delta) * w_level;
+        fvec<D + 1> w;  // b_r * w_level (:405), or dB[r] * w_level (:1244-1245)
+        if constexpr (kSecondOrder) {
+            w = pos_grad_grad_to_bary<D>(s.rank, q, scale_factor + level * D) * w_level;
+        } else {
+            w = barycentric<D>(s.rank, s.delta) * w_level;
+        }
         uvec<D + 1> slot;
         static_for<D + 1>(PENC_BODY(r) {
             PENC_INDEX(r);
@@ -195,6 +204,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
                                               streaming, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
         if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
         pos = pos_next;
+        q = q_next;
         g0 = g0_next;
         g1 = g1_next;
     }
@@ -254,84 +264,44 @@ reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size
 }
 
 // ------------------------------------------------------------------------------------------
-// double backward from d(loss)/d(position gradient): either half, or both in one pass
-// (EncodingGPU.cuh:1016-1257 scatter into the table gradient, 1260-1493 grad of grad_sliced)
+// double backward from d(loss)/d(position gradient), the half that gathers: gradient w.r.t.
+// grad_sliced_values (EncodingGPU.cuh:1260-1493).  One thread per (point, level), a level at a
+// time, like the forward.  (The other half, the scatter into the table gradient, is
+// backward_table_kernel<D, false, true>.  One kernel doing both, with eight tiles per workgroup,
+// was measured 7-13% slower than the two: the gathering half wants small workgroups, the scattering
+// half large groups of points with the levels interleaved.)
 
-template <int D, bool kTableGrad, bool kGradGrad>
-__global__ void __launch_bounds__(kScatterBlock)
-double_backward_kernel(int n_points, int n_levels, int first_level, int tiles_per_group, uint32_t interleaved_levels,
-                       uint32_t capacity, uint32_t cap_mask,
-                       const float* __restrict__ positions, const float* __restrict__ table,
-                       const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
-                       const float* __restrict__ window, const float* __restrict__ double_pos_grad,
-                       const float* __restrict__ grad_sliced, float* __restrict__ table_grad,
-                       float* __restrict__ grad_grad_sliced, BinTarget pass_bins) {
-    __shared__ ScatterState state;
-    // a level at a time (blockIdx.y) whenever the kernel gathers from the table: interleaving levels
-    // was then measured equal to 13% slower (the slices fall out of L2)
-    uint32_t level_in_pass = blockIdx.y, group = blockIdx.x;
-    if (interleaved_levels != 0u) {  // the table-gradient half on its own: dealt to the dies like backward_table_kernel
-        const uint32_t die = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
-        level_in_pass = j % interleaved_levels;
-        group = (j / interleaved_levels) * kXcds + die;
-        if (static_cast<int64_t>(group) * tiles_per_group * kScatterBlock >= n_points) return;
+template <int D>
+__global__ void __launch_bounds__(kBlock)
+grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
+                 const float* __restrict__ positions, const float* __restrict__ table,
+                 const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
+                 const float* __restrict__ window, const float* __restrict__ double_pos_grad,
+                 float* __restrict__ grad_grad_sliced) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= n_points) return;
+    const int level = blockIdx.y;
+    float* o = grad_grad_sliced + (static_cast<size_t>(level) * 2) * n_points + n;
+    const float w_level = level < n_levels ? window[level] : 0.0f;  // concat levels: zeros (:1290-1295)
+    if (w_level == 0.0f) {
+        o[0] = 0.0f;
+        o[n_points] = 0.0f;
+        return;
     }
-    const int level = first_level + level_in_pass;
-    const bool extra_level = level >= n_levels;  // concat levels: zeros (:1290-1295)
-    const float w_level = extra_level ? 0.0f : window[level];
-    const bool live = w_level != 0.0f;
-    if (!live && !kGradGrad) return;
-    if (kTableGrad && live) scatter_begin(state);
-    const int lvl = extra_level ? 0 : level;
-    const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
-    float* level_grad = kTableGrad ? table_grad + static_cast<size_t>(lvl) * capacity * 2 : nullptr;
-    const float* level_table = table + static_cast<size_t>(lvl) * capacity * 2;
-    const float* sf = scale_factor + lvl * D;
-    const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
-    const float* g1p = g0p + n_points;
-    bool streaming = false;
-    for (int t = 0; t < tiles_per_group; ++t) {
-        const int64_t tile_base = (static_cast<int64_t>(group) * tiles_per_group + t) * kScatterBlock;
-        if (tile_base >= n_points) break;
-        if (kTableGrad && live && !streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
-        const bool active = tile_base + threadIdx.x < n_points;
-        const int n = static_cast<int>(tile_base) + threadIdx.x;
-        const int nn = active ? n : n_points - 1;
-        float gg0 = 0.0f, gg1 = 0.0f;
-        if (live) {
-            const Located<D> s = locate<D>(load_point<D>(positions, nn), random_shift + lvl * D, sf);
-            const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
-            uvec<D + 1> slot;
-            static_for<D + 1>(PENC_BODY(r) {
-                PENC_INDEX(r);
-                slot[r] = to_slot(h[r], capacity, cap_mask);
-            });
-            Vertices<D> v;
-            if constexpr (kGradGrad) v = load_vertices<D>(level_table, h, capacity, cap_mask);
-            // dB[r] * w_level, then times g_f or times the vertex value (:1244-1245, :1484-1485)
-            const fvec<D + 1> wr = pos_grad_grad_to_bary<D>(s.rank, load_point<D>(double_pos_grad, nn), sf) * w_level;
-            // the scatter does not need the gathered table entries: it runs while they are in flight
-            if constexpr (kTableGrad) {
-                const float g0 = g0p[nn], g1 = g1p[nn];
-                const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
-                                                      streaming, slot, wr * g0, wr * g1);
-                if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
-            }
-            if constexpr (kGradGrad) {
-                static_for<D + 1>(PENC_BODY(r) {
-                    PENC_INDEX(r);
-                    gg0 += wr[r] * v.f0[r];
-                    gg1 += wr[r] * v.f1[r];
-                });
-            }
-        }
-        if (kGradGrad && active) {
-            float* o = grad_grad_sliced + (static_cast<size_t>(level) * 2) * n_points + n;
-            o[0] = gg0;
-            o[n_points] = gg1;
-        }
-    }
-    if (kTableGrad && live) scatter_end(state, level_grad, bins, group, streaming);
+    const float* sf = scale_factor + level * D;
+    const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, sf);
+    const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
+    const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
+    // dB[r] * w_level, then times the vertex value (:1484-1485)
+    const fvec<D + 1> wr = pos_grad_grad_to_bary<D>(s.rank, load_point<D>(double_pos_grad, n), sf) * w_level;
+    float gg0 = 0.0f, gg1 = 0.0f;
+    static_for<D + 1>(PENC_BODY(r) {
+        PENC_INDEX(r);
+        gg0 += wr[r] * v.f0[r];
+        gg1 += wr[r] * v.f1[r];
+    });
+    o[0] = gg0;
+    o[n_points] = gg1;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -445,7 +415,6 @@ inline uint32_t bins_for_capacity(int capacity) {
     return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
 }
 
-constexpr int kSplitDoubleBackwardMaxDim = 4;
 constexpr int64_t kMinSlotsPerContribution = 8;
 constexpr int64_t kLargeGroupsMinWorkgroups = 3000;  // about four per workgroup slot of the chip (256 CUs x 3)
 
@@ -549,11 +518,12 @@ using namespace penc;
 
 // The table gradient of penc_backward / penc_backward_table_rowmajor: clear, scatter, reduce the
 // bins, in as many passes over the levels as the workspace asks for.  grad_row_stride == 0 means
-// the [level][feature][n] layout, otherwise the gradient is rows of that many floats.
+// the [level][feature][n] layout, otherwise the gradient is rows of that many floats.  With
+// double_pos_grad the same for the table-gradient half of the double backward (level-major only).
 static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
                           const float* scale_factor, const float* random_shift, const float* anneal_window,
-                          const float* grad, int64_t grad_row_stride, float* lattice_values_grad, void* workspace,
-                          size_t workspace_bytes, hipStream_t st) {
+                          const float* grad, int64_t grad_row_stride, const float* double_pos_grad,
+                          float* lattice_values_grad, void* workspace, size_t workspace_bytes, hipStream_t st) {
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
@@ -564,15 +534,18 @@ static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int 
         const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
         const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
         const dim3 grid(padded_groups * static_cast<unsigned>(count));
-#define PENC_LAUNCH_TABLE(ROW_MAJOR)                                                                                       \
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR>), grid, dim3(kScatterBlock), 0, st, n, \
-                                                first, static_cast<uint32_t>(count), tiles_per_group, cap, mask, positions,  \
-                                                scale_factor, random_shift, anneal_window, grad, grad_row_stride,            \
-                                                lattice_values_grad, plan.target))
-        if (grad_row_stride != 0) {
-            PENC_LAUNCH_TABLE(true);
+#define PENC_LAUNCH_TABLE(ROW_MAJOR, SECOND_ORDER)                                                                         \
+    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER>), grid,                  \
+                                                dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
+                                                tiles_per_group, cap, mask, positions, scale_factor, random_shift,           \
+                                                anneal_window, grad, grad_row_stride, double_pos_grad, lattice_values_grad,  \
+                                                plan.target))
+        if (double_pos_grad != nullptr) {
+            PENC_LAUNCH_TABLE(false, true);
+        } else if (grad_row_stride != 0) {
+            PENC_LAUNCH_TABLE(true, false);
         } else {
-            PENC_LAUNCH_TABLE(false);
+            PENC_LAUNCH_TABLE(false, false);
         }
 #undef PENC_LAUNCH_TABLE
         if (int rc = check_launch()) return rc;
@@ -670,7 +643,7 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     if (lattice_values_grad)
         if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
-                                    anneal_window, grad_sliced_values, 0, lattice_values_grad, workspace, workspace_bytes, st))
+                                    anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, workspace, workspace_bytes, st))
             return rc;
     if (positions_grad) {
         // levels in groups of kPosLevelsPerGroup when the workspace can hold the partial sums
@@ -713,7 +686,7 @@ int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions,
         return PENC_ERR_BAD_SIZE;
     if (!aligned8(lattice_values_grad) || !aligned8(grad_rows)) return PENC_ERR_MISALIGNED;
     return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
-                          grad_rows, grad_row_stride, lattice_values_grad, workspace, workspace_bytes,
+                          grad_rows, grad_row_stride, nullptr, lattice_values_grad, workspace, workspace_bytes,
                           static_cast<hipStream_t>(stream));
 }
 
@@ -733,46 +706,18 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
     if (!lattice_values_grad && !grad_grad_sliced_values) return PENC_ERR_NULL_POINTER;
     if (!aligned8(lattice_values) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int n = static_cast<int>(nr_positions);
-    const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
-    const dim3 block(kScatterBlock);
-#define PENC_LAUNCH_DB(TG, GG, GRID, FIRST, TILES, INTERLEAVED, TARGET)                                               \
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((double_backward_kernel<DD, TG, GG>), GRID, block, 0, st, n, nr_levels,  \
-                                                FIRST, TILES, INTERLEAVED, cap, mask, positions, lattice_values,         \
-                                                scale_factor, random_shift, anneal_window, double_positions_grad,       \
-                                                grad_sliced_values, lattice_values_grad, grad_grad_sliced_values, TARGET))
-    // Both halves in one kernel share the simplex search, but the table-gradient half on its own can
-    // interleave levels and take large groups like backward_table_kernel.  Measured: two kernels are
-    // 2-9% faster up to D = 4 and 13% slower at D = 8, where the search is the expensive part.
-    const bool split = lattice_values_grad && grad_grad_sliced_values && pos_dim <= kSplitDoubleBackwardMaxDim;
-    const unsigned groups8 = scatter_groups(nr_positions, kScatterTiles);
-    if (grad_grad_sliced_values && (!lattice_values_grad || split)) {
-        PENC_LAUNCH_DB(false, true, dim3(groups8, nr_levels + extra), 0, kScatterTiles, 0u, BinTarget{});
+    if (grad_grad_sliced_values) {
+        const dim3 grid(tiles(nr_positions), nr_levels + extra);
+        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((grad_grad_kernel<DD>), grid, dim3(kBlock), 0, st,
+                                                    static_cast<int>(nr_positions), nr_levels,
+                                                    static_cast<uint32_t>(capacity), mask_of(capacity), positions,
+                                                    lattice_values, scale_factor, random_shift, anneal_window,
+                                                    double_positions_grad, grad_grad_sliced_values));
         if (int rc = check_launch()) return rc;
-        if (!lattice_values_grad) return PENC_OK;
     }
-    const bool alone = !grad_grad_sliced_values || split;  // the table-gradient half runs without the gathers
-    const int tiles_per_group = alone ? table_backward_tiles(nr_positions, nr_levels) : kScatterTiles;
-    if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, tiles_per_group, workspace, workspace_bytes);
-    const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
-    for (int first = 0; first < nr_levels; first += per_pass) {
-        int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
-        const int scatter_levels = count;
-        if (alone) {
-            const unsigned padded = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
-            PENC_LAUNCH_DB(true, false, dim3(padded * static_cast<unsigned>(count)), first, tiles_per_group,
-                           static_cast<uint32_t>(count), plan.target);
-        } else {
-            if (first + count == nr_levels) count += extra;  // the zero-filled concat levels
-            PENC_LAUNCH_DB(true, true, dim3(groups8, count), first, kScatterTiles, 0u, plan.target);
-        }
-        if (int rc = check_launch()) return rc;
-        if (plan.enabled)
-            if (int rc = reduce_bins(plan, anneal_window, first, scatter_levels, capacity, lattice_values_grad, st)) return rc;
-    }
-#undef PENC_LAUNCH_DB
-    return PENC_OK;
+    if (!lattice_values_grad) return PENC_OK;
+    return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
+                          grad_sliced_values, 0, double_positions_grad, lattice_values_grad, workspace, workspace_bytes, st);
 }
 
 int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream) {
