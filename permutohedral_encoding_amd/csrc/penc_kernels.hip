@@ -23,10 +23,9 @@
 
 namespace penc {
 
-#ifndef PENC_POS_LEVELS_PER_GROUP
-#define PENC_POS_LEVELS_PER_GROUP 2
-#endif
-constexpr int kPosLevelsPerGroup = PENC_POS_LEVELS_PER_GROUP;  // levels one position-gradient thread sums
+// Levels one position-gradient thread sums in registers (measured: 2 is fastest up to D = 5, 1
+// from D = 6 on, where a thread's arithmetic per level is long enough; 3 and 4 are slower everywhere).
+constexpr int pos_levels_per_group(int pos_dim) { return pos_dim >= 6 ? 1 : 2; }
 
 constexpr int kDefaultLevelsPerPass = 1 << 20;  // by default the suggested workspace bins all levels in one pass (measured fastest)
 
@@ -592,8 +591,8 @@ size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_le
 }
 
 size_t penc_positions_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels) {
-    if (pos_dim < 2 || pos_dim > 8 || nr_positions <= 0 || nr_levels <= kPosLevelsPerGroup) return 0;
-    const size_t groups = static_cast<size_t>((nr_levels + kPosLevelsPerGroup - 1) / kPosLevelsPerGroup);
+    if (pos_dim < 2 || pos_dim > 8 || nr_positions <= 0 || nr_levels <= pos_levels_per_group(pos_dim)) return 0;
+    const size_t groups = static_cast<size_t>((nr_levels + pos_levels_per_group(pos_dim) - 1) / pos_levels_per_group(pos_dim));
     return groups * static_cast<size_t>(nr_positions) * pos_dim * sizeof(float) + 256;
 }
 
@@ -646,16 +645,16 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                                     anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, workspace, workspace_bytes, st))
             return rc;
     if (positions_grad) {
-        // levels in groups of kPosLevelsPerGroup when the workspace can hold the partial sums
+        // levels in groups of pos_levels_per_group() when the workspace can hold the partial sums
         // (the table-gradient scatter above is done with it: same stream), else one group
         const size_t n_values = static_cast<size_t>(nr_positions) * pos_dim;
         int per_group = nr_levels, groups = 1;
         float* partial = positions_grad;
         const uintptr_t ws = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
-        const int want_groups = (nr_levels + kPosLevelsPerGroup - 1) / kPosLevelsPerGroup;
+        const int want_groups = (nr_levels + pos_levels_per_group(pos_dim) - 1) / pos_levels_per_group(pos_dim);
         if (workspace != nullptr && want_groups > 1 &&
             workspace_bytes >= (ws - reinterpret_cast<uintptr_t>(workspace)) + want_groups * n_values * sizeof(float)) {
-            per_group = kPosLevelsPerGroup;
+            per_group = pos_levels_per_group(pos_dim);
             groups = want_groups;
             partial = reinterpret_cast<float*>(ws);
         }
