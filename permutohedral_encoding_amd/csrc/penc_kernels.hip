@@ -24,7 +24,8 @@
 namespace penc {
 
 // Levels one position-gradient thread sums in registers (measured: 2 is fastest up to D = 5, 1
-// from D = 6 on, where a thread's arithmetic per level is long enough; 3 and 4 are slower everywhere).
+// from D = 6 on, where a thread's arithmetic per level is long enough; 3 and 4 are slower everywhere,
+// also with all their gathers issued up front: more levels at a time overflow L2).
 constexpr int pos_levels_per_group(int pos_dim) { return pos_dim >= 6 ? 1 : 2; }
 
 constexpr int kDefaultLevelsPerPass = 1 << 20;  // by default the suggested workspace bins all levels in one pass (measured fastest)
