@@ -29,6 +29,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 #include "penc_lattice.hpp"
@@ -45,7 +46,7 @@ constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
 constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space
-constexpr int kStageChunk = 4;         // vertices per thread a wave sorts by bin in one go (256 records)
+constexpr int kStageChunk = 5;         // vertices per thread a wave sorts by bin in one go (320 records)
 constexpr int kStageBins = 64;         // a wave counts one bin per lane: staging needs n_bins <= 64
 constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
@@ -163,6 +164,8 @@ __device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad,
 struct ScatterState {
     int tag[kCacheLines];
     double val[kCacheLines][2];
+    // when the workgroup streams, val and this tail together are its waves' staging slices
+    uint4 stage_tail[(kScatterBlock / 64) * kStageChunk * 64 - kCacheLines];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
     uint32_t hits;                 // contributions the cache has absorbed into existing lines
 };
@@ -221,7 +224,7 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
 }
 
 // Stage 2 for a whole tile once the workgroup streams (see scatter_stream_switch): the cache's LDS
-// is staging space, a 4 KiB slice per wave.  For kStageChunk vertices per thread at a time, the wave
+// is staging space, a 5 KiB slice per wave.  For kStageChunk vertices per thread at a time, the wave
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
 // its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
@@ -233,7 +236,9 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
                                             fvec<D + 1> a1) {
     constexpr int kWaves = kScatterBlock / 64;
     static_assert(kCacheLines / kWaves >= 4 * 64, "four 64-entry arrays per wave live in the tag array");
-    static_assert(sizeof(c.val) / kWaves >= kStageChunk * 64 * sizeof(uint4), "staging slice of a wave");
+    static_assert(offsetof(ScatterState, stage_tail) == offsetof(ScatterState, val) + sizeof(c.val) &&
+                      (sizeof(c.val) + sizeof(c.stage_tail)) / kWaves == kStageChunk * 64 * sizeof(uint4),
+                  "val and stage_tail are one contiguous array of staging slices");
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     uint32_t* count = reinterpret_cast<uint32_t*>(c.tag) + wave * (kCacheLines / kWaves);  // records per bin
     uint32_t* offset = count + 64;  // where a bin's run starts in the wave's slice
