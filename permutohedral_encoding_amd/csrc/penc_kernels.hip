@@ -290,10 +290,16 @@ grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mas
     }
     const float* sf = scale_factor + level * D;
     const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, sf);
-    const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
+    // one trip through the thread's LDS column puts both the elevated gradient and the hash steps
+    // into rank order (as in the forward)
+    __shared__ uint2 columns[(D + 1) * kBlock];
+    uvec<D + 1> h;
+    fvec<D + 1> sorted;
+    sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, pos_grad_grad_to_elevated<D>(load_point<D>(double_pos_grad, n), sf),
+                        s.hash0, sorted, h);
     const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
     // dB[r] * w_level, then times the vertex value (:1484-1485)
-    const fvec<D + 1> wr = pos_grad_grad_to_bary<D>(s.rank, load_point<D>(double_pos_grad, n), sf) * w_level;
+    const fvec<D + 1> wr = sorted_elevated_grad_to_bary<D>(sorted) * w_level;
     float gg0 = 0.0f, gg1 = 0.0f;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);

@@ -314,10 +314,11 @@ __device__ __forceinline__ fvec<D> bary_grad_to_pos_grad(ivec<D + 1> rank, fvec<
     return elevated_grad_to_pos_grad<D>(pick_by_rank<D>(rank, bary_grad_by_rank<D>(dB)), sf);
 }
 
-// d(loss)/d(position gradient) -> derivative w.r.t. each vertex weight (EncodingGPU.cuh:1187-1218).
+// d(loss)/d(position gradient) -> derivative w.r.t. each vertex weight (EncodingGPU.cuh:1187-1218),
+// in two steps with the permutation into rank order between them.
+// Step 1: the derivative w.r.t. the elevated coordinates, already divided by D+1.
 template <int D>
-__device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_bary(ivec<D + 1> rank, fvec<D> q,
-                                                             const float* __restrict__ sf) {
+__device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_elevated(fvec<D> q, const float* __restrict__ sf) {
     constexpr int D1 = D + 1;
     constexpr float kInv = 1.0f / D1;
     fvec<D> g;
@@ -344,8 +345,14 @@ __device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_bary(ivec<D + 1> rank, f
         dE[j] -= g[j - 1] * static_cast<float>(j);
     });
     dE *= kInv;
-    const fvec<D1> sorted = by_rank<D>(rank, dE);
-    // dB[k] = sorted[D-k] - sorted[D+1-k]; dB[D+1] = -sorted[0] is folded into dB[0] (:1218)
+    return dE;
+}
+
+// Step 2, from dE in rank order: dB[k] = sorted[D-k] - sorted[D+1-k]; dB[D+1] = -sorted[0] is folded
+// into dB[0] (:1218).
+template <int D>
+__device__ __forceinline__ fvec<D + 1> sorted_elevated_grad_to_bary(fvec<D + 1> sorted) {
+    constexpr int D1 = D + 1;
     fvec<D1> dB;
     dB[0] = sorted[D] + (0.0f - sorted[0]);
     static_for<D>(PENC_BODY(rr) {
@@ -354,6 +361,12 @@ __device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_bary(ivec<D + 1> rank, f
         dB[r] = sorted[D - r] - sorted[D1 - r];
     });
     return dB;
+}
+
+template <int D>
+__device__ __forceinline__ fvec<D + 1> pos_grad_grad_to_bary(ivec<D + 1> rank, fvec<D> q,
+                                                             const float* __restrict__ sf) {
+    return sorted_elevated_grad_to_bary<D>(by_rank<D>(rank, pos_grad_grad_to_elevated<D>(q, sf)));
 }
 
 }  // namespace penc
