@@ -415,3 +415,38 @@ def test_many_bins_and_few_contributions_per_slot():
         tg, _ = enc.backward(inp, to_gpu(p["grad"]))
         want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
         assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, {n} points")
+
+
+@pytest.mark.parametrize("d", [2, 5, 6, 7])
+def test_large_size_identities_in_the_other_dimensions(d):
+    """The benchmark configurations cover D = 3, 4, 8 at full size; the same size-independent checks for
+    the remaining dimensions, at sizes where the large point groups and interleaved levels are in use:
+    adjoint identities, and every slot of the binned table gradients against the direct-atomics path."""
+    from permutohedral_encoding_amd import _native
+    n, levels, cap = 1 << 19, 16, 1 << 18
+    p = random_problem(d, n, levels, cap, seed=50 + d, sigma_range=(1.0, 1e-3))
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p)
+    grad_t, dpos_t = to_gpu(p["grad"]), to_gpu(p["dpos"])
+    table = inp.m_lattice_values.double()
+    out = enc.forward(inp)
+    tg, pg = enc.backward(inp, grad_t)
+    tg2, ggs = enc.double_backward_from_positions(inp, dpos_t, grad_t)
+    lhs = torch.sum(out.double() * grad_t.double()).item()
+    rhs = torch.sum(tg.double() * table).item()
+    scale = torch.sum(torch.abs(out.double() * grad_t.double())).item()
+    assert abs(lhs - rhs) <= 1e-5 * scale, (lhs, rhs, scale)
+    a = torch.sum(dpos_t.double() * pg.double()).item()
+    b = torch.sum(ggs.double() * grad_t.double()).item()
+    c = torch.sum(tg2.double() * table).item()
+    scale2 = torch.sum(torch.abs(ggs.double() * grad_t.double())).item()
+    assert abs(a - b) <= 1e-4 * scale2 and abs(a - c) <= 1e-4 * scale2, (a, b, c, scale2)
+    saved = _native.LEVELS_PER_PASS
+    _native.LEVELS_PER_PASS = -1
+    try:
+        tg_direct, _ = enc.backward(inp, grad_t)
+        tg2_direct, _ = enc.double_backward_from_positions(inp, dpos_t, grad_t)
+    finally:
+        _native.LEVELS_PER_PASS = saved
+    assert torch.allclose(tg, tg_direct, rtol=1e-3, atol=1e-5 * tg.abs().max().item())
+    assert torch.allclose(tg2, tg2_direct, rtol=1e-3, atol=1e-5 * tg2.abs().max().item())
