@@ -50,6 +50,7 @@ extern "C" {
 #define PENC_ERR_UNSUPPORTED_NR_FEAT 4 /* nr_feat != 2 (reference: Encoding.cuh:142) */
 #define PENC_ERR_MISALIGNED 5          /* lattice_values / lattice_values_grad not 8-byte aligned */
 #define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
+#define PENC_ERR_SCRATCH_TOO_SMALL 7    /* penc_backward_static: the problem does not fit the static scratch */
 
 const char* penc_status_string(int status);
 
@@ -96,6 +97,28 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* random_shift, const float* anneal_window,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                   void* workspace, size_t workspace_bytes, void* stream);
+
+/* penc_backward for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as penc_backward without the workspace: the scratch the table-gradient
+ * scatter and the position-gradient partial sums use is a fixed array of
+ * PENC_STATIC_SCRATCH_BYTES inside the library's code object (one copy per GPU, held until the
+ * process ends).  The call allocates and frees nothing.
+ *   - Limit: one level's slot-range records must fit, i.e.
+ *     penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels, capacity, 1) <= PENC_STATIC_SCRATCH_BYTES
+ *     (about 1.2 million points at pos_dim 3); larger problems return PENC_ERR_SCRATCH_TOO_SMALL
+ *     and nothing is enqueued.  Levels are binned in as many passes as the scratch needs; position
+ *     gradients whose partial sums do not fit are summed by one thread per point instead.
+ *   - Every call on a GPU uses that GPU's one array, whose contents survive between calls; nothing
+ *     in it has to start at zero (every count is written before it is read).  Calls that overlap on
+ *     one GPU (two streams, two threads) race on it: serialise them. */
+#define PENC_STATIC_SCRATCH_BYTES (64u << 20)
+size_t penc_static_scratch_bytes(void);
+int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                         const float* positions, const float* lattice_values, const float* scale_factor,
+                         const float* random_shift, const float* anneal_window,
+                         const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
+                         void* stream);
 
 /* The table gradient of penc_backward, reading the upstream gradient as the layer after the encoding
  * produces it: rows grad_rows[n][2*level + feature] of grad_row_stride floats (even, >= 2*nr_levels;

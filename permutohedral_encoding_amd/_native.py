@@ -31,6 +31,10 @@ _SIGNATURES = {
     "penc_backward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                      _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                      ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_static_scratch_bytes": (ctypes.c_size_t, []),
+    "penc_backward_static": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                            ctypes.c_void_p]),
     "penc_backward_table_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                                     _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
                                                     ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),

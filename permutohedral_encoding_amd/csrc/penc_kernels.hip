@@ -17,6 +17,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "../../include/penc.h"
 #include "penc_lattice.hpp"
 #include "penc_scatter.hpp"
@@ -374,6 +376,14 @@ __global__ void __launch_bounds__(kBlock) fill_zero_kernel(float2* __restrict__ 
 }
 
 // ------------------------------------------------------------------------------------------
+// Scratch of penc_backward_static: device memory that is part of the loaded code object, so that
+// callers who must not allocate (HIP graph capture, serving loops) still get the binned scatter.
+// Every GPU the library runs on holds its own copy until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress: its device address is looked up once per
+// device (static_scratch_of) and that pointer is what the launchers pass on.
+static __device__ __align__(256) unsigned char scratch[PENC_STATIC_SCRATCH_BYTES];
+
+// ------------------------------------------------------------------------------------------
 // host side
 
 inline int check_launch() { return hipGetLastError() == hipSuccess ? PENC_OK : PENC_ERR_LAUNCH; }
@@ -518,6 +528,26 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
 
 inline unsigned tiles(int64_t n) { return static_cast<unsigned>((n + kBlock - 1) / kBlock); }
 
+// Device address of this GPU's copy of `scratch`, looked up on the first call with that GPU
+// current and kept for the life of the process.  Returns nullptr when the lookup fails.
+constexpr int kMaxDevices = 64;
+inline void* static_scratch_of_current_device() {
+    static std::mutex lock;
+    static void* address[kMaxDevices] = {};
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> guard(lock);
+    if (address[device] == nullptr) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();  // the failure is reported by the caller's status code, not by a later launch check
+            return nullptr;
+        }
+        address[device] = p;
+    }
+    return address[device];
+}
+
 }  // namespace penc
 
 using namespace penc;
@@ -561,6 +591,55 @@ static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int 
     return PENC_OK;
 }
 
+// penc_backward and penc_backward_static: argument checks, then the table gradient (clear, scatter,
+// reduce) and the position gradient on the same stream.
+static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                         const float* positions, const float* lattice_values, const float* scale_factor,
+                         const float* random_shift, const float* anneal_window,
+                         const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
+                         void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
+    if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_sliced_values)
+        return PENC_ERR_NULL_POINTER;
+    if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
+    if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
+    if ((lattice_values && !aligned8(lattice_values)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int n = static_cast<int>(nr_positions);
+    const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
+    if (lattice_values_grad)
+        if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+                                    anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, workspace, workspace_bytes, st))
+            return rc;
+    if (positions_grad) {
+        // levels in groups of pos_levels_per_group() when the workspace can hold the partial sums
+        // (the table-gradient scatter above is done with it: same stream), else one group
+        const size_t n_values = static_cast<size_t>(nr_positions) * pos_dim;
+        int per_group = nr_levels, groups = 1;
+        float* partial = positions_grad;
+        const uintptr_t ws = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
+        const int want_groups = (nr_levels + pos_levels_per_group(pos_dim) - 1) / pos_levels_per_group(pos_dim);
+        if (workspace != nullptr && want_groups > 1 &&
+            workspace_bytes >= (ws - reinterpret_cast<uintptr_t>(workspace)) + want_groups * n_values * sizeof(float)) {
+            per_group = pos_levels_per_group(pos_dim);
+            groups = want_groups;
+            partial = reinterpret_cast<float*>(ws);
+        }
+        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions), groups),
+                                                    dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
+                                                    lattice_values, scale_factor, random_shift, anneal_window,
+                                                    grad_sliced_values, partial));
+        if (int rc = check_launch()) return rc;
+        if (groups > 1) {
+            const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
+            hipLaunchKernelGGL(reduce_level_groups_kernel, dim3(static_cast<unsigned>(want < 8192 ? want : 8192)), dim3(kBlock),
+                               0, st, partial, groups, n_values, positions_grad);
+            if (int rc = check_launch()) return rc;
+        }
+    }
+    return PENC_OK;
+}
+
 extern "C" {
 
 const char* penc_status_string(int status) {
@@ -572,6 +651,7 @@ const char* penc_status_string(int status) {
         case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2 since other values are not implemented";
         case PENC_ERR_MISALIGNED: return "lattice_values and lattice_values_grad must be 8-byte aligned";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
+        case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
         default: return "unknown status";
     }
 }
@@ -638,46 +718,29 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* random_shift, const float* anneal_window,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                   void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+                         random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad, workspace,
+                         workspace_bytes, stream);
+}
+
+size_t penc_static_scratch_bytes(void) { return PENC_STATIC_SCRATCH_BYTES; }
+
+int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                         const float* positions, const float* lattice_values, const float* scale_factor,
+                         const float* random_shift, const float* anneal_window,
+                         const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
+                         void* stream) {
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
-    if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_sliced_values)
-        return PENC_ERR_NULL_POINTER;
-    if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
-    if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
-    if ((lattice_values && !aligned8(lattice_values)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const int n = static_cast<int>(nr_positions);
-    const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
-    if (lattice_values_grad)
-        if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
-                                    anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, workspace, workspace_bytes, st))
-            return rc;
-    if (positions_grad) {
-        // levels in groups of pos_levels_per_group() when the workspace can hold the partial sums
-        // (the table-gradient scatter above is done with it: same stream), else one group
-        const size_t n_values = static_cast<size_t>(nr_positions) * pos_dim;
-        int per_group = nr_levels, groups = 1;
-        float* partial = positions_grad;
-        const uintptr_t ws = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
-        const int want_groups = (nr_levels + pos_levels_per_group(pos_dim) - 1) / pos_levels_per_group(pos_dim);
-        if (workspace != nullptr && want_groups > 1 &&
-            workspace_bytes >= (ws - reinterpret_cast<uintptr_t>(workspace)) + want_groups * n_values * sizeof(float)) {
-            per_group = pos_levels_per_group(pos_dim);
-            groups = want_groups;
-            partial = reinterpret_cast<float*>(ws);
-        }
-        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions), groups),
-                                                    dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
-                                                    lattice_values, scale_factor, random_shift, anneal_window,
-                                                    grad_sliced_values, partial));
-        if (int rc = check_launch()) return rc;
-        if (groups > 1) {
-            const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
-            hipLaunchKernelGGL(reduce_level_groups_kernel, dim3(static_cast<unsigned>(want < 8192 ? want : 8192)), dim3(kBlock),
-                               0, st, partial, groups, n_values, positions_grad);
-            if (int rc = check_launch()) return rc;
-        }
-    }
-    return PENC_OK;
+    // the scratch must hold the slot-range records of at least one level (more levels per pass as
+    // they fit); a capacity the scatter does not bin needs no scratch at all
+    if (lattice_values_grad != nullptr &&
+        penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels, capacity, 1) > PENC_STATIC_SCRATCH_BYTES)
+        return PENC_ERR_SCRATCH_TOO_SMALL;
+    void* ws = static_scratch_of_current_device();
+    if (ws == nullptr) return PENC_ERR_LAUNCH;
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+                         random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad, ws,
+                         PENC_STATIC_SCRATCH_BYTES, stream);
 }
 
 int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
