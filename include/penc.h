@@ -155,10 +155,13 @@ int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* s
  *   rem0, rank : the remainder-0 lattice point and the residual ranks after the hyperplane wrap
  *   slot       : hashed table index of each of the D+1 vertices
  *   barycentric: the D+1 interpolation weights
- * Uses the same device code as the kernels above (reference: EncodingGPU.cuh:130-223). */
+ * The kernels share one routine for rem0 and rank and have two equivalent routines for slots and
+ * weights; gather_path picks which one is reported: 0 = the compare-and-select chains of the
+ * scattering and position-gradient kernels, 1 = the rank sort through LDS of the forward and
+ * grad-of-grad kernels (reference: EncodingGPU.cuh:130-223). */
 int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
                        const float* positions, const float* scale_factor, const float* random_shift,
-                       int* rem0, int* rank, int* slot, float* barycentric, void* stream);
+                       int gather_path, int* rem0, int* rank, int* slot, float* barycentric, void* stream);
 
 /* Memory-system probes used by the benchmark to measure the rooflines the encoding is priced
  * against; they have no counterpart in the reference.

@@ -134,7 +134,8 @@ def backward_table(pos, sf, shift, window, grad, capacity, dtype=np.float32, wan
 
 
 def backward_pos(pos, table, sf, shift, window, grad, dtype=np.float32):
-    """Returns dict(grad32=(N,D), grad64=(N,D) fp64-accumulated over levels)."""
+    """Returns dict(grad32=(N,D), grad64=(N,D) fp64-accumulated over levels, abs64=(N,D) the same chain
+    with every term replaced by its magnitude: the scale the rounding error of grad32 is relative to)."""
     pos, table, sf, shift, window, grad = (_f(a, dtype) for a in (pos, table, sf, shift, window, grad))
     n, d, l = _dims(pos, shift)
     c = table.shape[1]
@@ -145,14 +146,16 @@ def backward_pos(pos, table, sf, shift, window, grad, dtype=np.float32):
         return dict(grad64=g)
     g32 = np.empty(pos.shape, np.float32)
     g64 = np.empty(pos.shape, np.float64)
+    a64 = np.empty(pos.shape, np.float64)
     _check(lib().penc_oracle_backward_pos(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(grad),
-                                          _p(g32), _p(g64)), "backward_pos")
-    return dict(grad32=g32, grad64=g64)
+                                          _p(g32), _p(g64), _p(a64)), "backward_pos")
+    return dict(grad32=g32, grad64=g64, abs64=a64)
 
 
 def double_backward(pos, table, sf, shift, window, double_pos_grad, grad, concat_points=False, dtype=np.float32,
                     want32=True, want64=True, want_abs=False):
-    """Returns dict(grad32/grad64/abs64 = table gradient (L,C,2), ggs = (L+extra,2,N))."""
+    """Returns dict(grad32/grad64/abs64 = table gradient (L,C,2), ggs = (L+extra,2,N), and with want_abs
+    ggs_abs64 = the grad-of-grad chain with every term replaced by its magnitude)."""
     pos, table, sf, shift, window, q, grad = (_f(a, dtype) for a in (pos, table, sf, shift, window, double_pos_grad, grad))
     n, d, l = _dims(pos, shift)
     c = table.shape[1]
@@ -167,7 +170,9 @@ def double_backward(pos, table, sf, shift, window, double_pos_grad, grad, concat
     g32 = np.zeros((l, c, 2), np.float32) if want32 else None
     g64 = np.zeros((l, c, 2), np.float64) if want64 else None
     a64 = np.zeros((l, c, 2), np.float64) if want_abs else None
+    ga64 = np.empty(ggs.shape, np.float64) if want_abs else None
     _check(lib().penc_oracle_double_backward(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(q),
-                                             _p(grad), _p(g32), _p(g64), _p(a64), _p(ggs), int(bool(concat_points))),
+                                             _p(grad), _p(g32), _p(g64), _p(a64), _p(ggs), _p(ga64),
+                                             int(bool(concat_points))),
            "double_backward")
-    return dict(grad32=g32, grad64=g64, abs64=a64, ggs=ggs)
+    return dict(grad32=g32, grad64=g64, abs64=a64, ggs=ggs, ggs_abs64=ga64)

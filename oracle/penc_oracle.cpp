@@ -156,6 +156,27 @@ inline void double_backward_bary(const Simplex<D, R>& s, const R* q, const R* sf
     dB[0] += dB[D1];
 }
 
+// The chain of double_backward_bary with every term replaced by its magnitude: an upper bound of
+// the sum of |terms| behind each dB[k], the scale its rounding error is relative to.
+template <int D, typename R, typename A>
+inline void double_backward_bary_magnitude(const Simplex<D, R>& s, const R* q, const R* sf, A* mB /*[D+2]*/) {
+    constexpr int D1 = D + 1;
+    const A inv = static_cast<A>(1) / static_cast<A>(D1);
+    A mE[D1];
+    for (int j = 0; j <= D; ++j) mE[j] = 0;
+    for (int i = 0; i < D; ++i) {
+        const A g = std::fabs(static_cast<A>(q[i]) * static_cast<A>(sf[i]));
+        for (int j = 0; j <= i; ++j) mE[j] += g;
+        mE[i + 1] += g * static_cast<A>(i + 1);
+    }
+    for (int k = 0; k <= D1; ++k) mB[k] = 0;
+    for (int i = 0; i <= D; ++i) {
+        mB[D - s.rank[i]] += mE[i] * inv;
+        mB[D1 - s.rank[i]] += mE[i] * inv;
+    }
+    mB[0] += mB[D1];
+}
+
 inline int extra_levels(int pos_dim, int concat_points) {
     // src/Encoding.cu:71-74 with val_dim = 2
     return concat_points ? (pos_dim + 1) / 2 : 0;
@@ -295,14 +316,14 @@ void backward_table(int64_t N, int L, int C, const R* pos, const R* sf, const R*
 
 template <int D, typename R, typename A>
 void backward_pos(int64_t N, int L, int C, const R* pos, const R* table, const R* sf, const R* shift,
-                  const R* window, const R* grad, R* pgrad, A* pgrad_acc) {
+                  const R* window, const R* grad, R* pgrad, A* pgrad_acc, A* pgrad_abs) {
     constexpr int D1 = D + 1;
     const R inv = static_cast<R>(1) / static_cast<R>(D1);
 #pragma omp parallel for schedule(static)
     for (int64_t n = 0; n < N; ++n) {
         R sum[D];
-        A sum_acc[D];
-        for (int i = 0; i < D; ++i) { sum[i] = 0; sum_acc[i] = 0; }
+        A sum_acc[D], sum_abs[D];
+        for (int i = 0; i < D; ++i) { sum[i] = 0; sum_acc[i] = 0; sum_abs[i] = 0; }
         for (int l = 0; l < L; ++l) {
             const R w_lvl = window[l];
             const R* tl = table + static_cast<int64_t>(l) * C * 2;
@@ -312,32 +333,42 @@ void backward_pos(int64_t N, int L, int C, const R* pos, const R* table, const R
             const R g0 = grad[(static_cast<int64_t>(l) * 2 + 0) * N + n];
             const R g1 = grad[(static_cast<int64_t>(l) * 2 + 1) * N + n];
             R dB[D + 2];
-            for (int k = 0; k <= D1; ++k) dB[k] = 0;
+            A mB[D + 2];  // the same chain with every term replaced by its magnitude (the scale rounding errors are relative to)
+            for (int k = 0; k <= D1; ++k) { dB[k] = 0; mB[k] = 0; }
             for (int r = 0; r <= D; ++r) {
                 int key[D1];
                 vertex_key<D, R>(s, r, key);
                 const int64_t h = 2 * static_cast<int64_t>(lattice_slot<D>(key, C));
                 dB[r] += tl[h] * w_lvl * g0;
                 dB[r] += tl[h + 1] * w_lvl * g1;
+                mB[r] = std::fabs(static_cast<A>(tl[h] * w_lvl * g0)) + std::fabs(static_cast<A>(tl[h + 1] * w_lvl * g1));
             }
             dB[D1] += dB[0];  // ":698"
+            mB[D1] = mB[0];
             R dE[D1];
+            A mE[D1];
             for (int i = 0; i <= D; ++i) {
                 dE[i] = 0;
                 dE[i] += dB[D - s.rank[i]] * inv;
                 dE[i] -= dB[D1 - s.rank[i]] * inv;
+                mE[i] = (mB[D - s.rank[i]] + mB[D1 - s.rank[i]]) * static_cast<A>(inv);
             }
             for (int i = 0; i < D; ++i) {
                 R dP = 0;
+                A mP = 0;
                 for (int j = 0; j <= i; ++j) dP += dE[j] * sfl[i];
+                for (int j = 0; j <= i; ++j) mP += mE[j] * std::fabs(static_cast<A>(sfl[i]));
                 dP -= dE[i + 1] * sfl[i] * static_cast<R>(i + 1);
+                mP += mE[i + 1] * std::fabs(static_cast<A>(sfl[i])) * static_cast<A>(i + 1);
                 sum[i] += dP;
                 sum_acc[i] += static_cast<A>(dP);
+                sum_abs[i] += mP;
             }
         }
         for (int i = 0; i < D; ++i) {
             if (pgrad) pgrad[n * D + i] = sum[i];
             if (pgrad_acc) pgrad_acc[n * D + i] = sum_acc[i];
+            if (pgrad_abs) pgrad_abs[n * D + i] = sum_abs[i];
         }
     }
 }
@@ -351,7 +382,7 @@ void backward_pos(int64_t N, int L, int C, const R* pos, const R* table, const R
 template <int D, typename R, typename A>
 void double_backward(int64_t N, int L, int C, const R* pos, const R* table, const R* sf, const R* shift,
                      const R* window, const R* q, const R* grad, R* tgrad, A* tgrad_acc, A* tgrad_abs,
-                     R* ggs, int concat_points) {
+                     R* ggs, A* ggs_abs, int concat_points) {
     constexpr int D1 = D + 1;
     const int extra = extra_levels(D, concat_points);
     for (int l = 0; l < L; ++l) {
@@ -363,6 +394,9 @@ void double_backward(int64_t N, int L, int C, const R* pos, const R* table, cons
             locate_simplex<D, R>(pos + n * D, shift + l * D, sf + l * D, s);
             R dB[D + 2];
             double_backward_bary<D, R>(s, q + n * D, sf + l * D, dB);
+            A mB[D + 2];
+            if (ggs_abs) double_backward_bary_magnitude<D, R, A>(s, q + n * D, sf + l * D, mB);
+            A ma0 = 0, ma1 = 0;
             const R g0 = grad[(static_cast<int64_t>(l) * 2 + 0) * N + n];
             const R g1 = grad[(static_cast<int64_t>(l) * 2 + 1) * N + n];
             R gg0 = 0, gg1 = 0;
@@ -393,15 +427,24 @@ void double_backward(int64_t N, int L, int C, const R* pos, const R* table, cons
                     gg0 += dB[r] * w_lvl * table[h];
                     gg1 += dB[r] * w_lvl * table[h + 1];
                 }
+                if (ggs_abs) {
+                    ma0 += mB[r] * std::fabs(static_cast<A>(w_lvl)) * std::fabs(static_cast<A>(table[h]));
+                    ma1 += mB[r] * std::fabs(static_cast<A>(w_lvl)) * std::fabs(static_cast<A>(table[h + 1]));
+                }
             }
             if (ggs) {
                 ggs[(static_cast<int64_t>(l) * 2 + 0) * N + n] = gg0;
                 ggs[(static_cast<int64_t>(l) * 2 + 1) * N + n] = gg1;
             }
+            if (ggs_abs) {
+                ggs_abs[(static_cast<int64_t>(l) * 2 + 0) * N + n] = ma0;
+                ggs_abs[(static_cast<int64_t>(l) * 2 + 1) * N + n] = ma1;
+            }
         }
     }
-    if (ggs) {
-        for (int64_t k = static_cast<int64_t>(L) * 2 * N; k < static_cast<int64_t>(L + extra) * 2 * N; ++k) ggs[k] = 0;
+    for (int64_t k = static_cast<int64_t>(L) * 2 * N; k < static_cast<int64_t>(L + extra) * 2 * N; ++k) {
+        if (ggs) ggs[k] = 0;
+        if (ggs_abs) ggs_abs[k] = 0;
     }
 }
 
@@ -506,9 +549,9 @@ int penc_oracle_backward_table_f64(int pos_dim, int64_t N, int L, int C, const d
 
 int penc_oracle_backward_pos(int pos_dim, int64_t N, int L, int C, const float* pos, const float* table,
                              const float* sf, const float* shift, const float* window, const float* grad,
-                             float* pgrad, double* pgrad_acc64) {
+                             float* pgrad, double* pgrad_acc64, double* pgrad_abs64) {
     if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (backward_pos<DD, float, double>(N, L, C, pos, table, sf, shift, window, grad, pgrad, pgrad_acc64)));
+    DISPATCH_D(pos_dim, (backward_pos<DD, float, double>(N, L, C, pos, table, sf, shift, window, grad, pgrad, pgrad_acc64, pgrad_abs64)));
     return 0;
 }
 
@@ -516,16 +559,17 @@ int penc_oracle_backward_pos_f64(int pos_dim, int64_t N, int L, int C, const dou
                                  const double* sf, const double* shift, const double* window,
                                  const double* grad, double* pgrad) {
     if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (backward_pos<DD, double, double>(N, L, C, pos, table, sf, shift, window, grad, pgrad, nullptr)));
+    DISPATCH_D(pos_dim, (backward_pos<DD, double, double>(N, L, C, pos, table, sf, shift, window, grad, pgrad, nullptr, nullptr)));
     return 0;
 }
 
 int penc_oracle_double_backward(int pos_dim, int64_t N, int L, int C, const float* pos, const float* table,
                                 const float* sf, const float* shift, const float* window,
                                 const float* double_pos_grad, const float* grad, float* tgrad,
-                                double* tgrad_acc64, double* tgrad_abs64, float* ggs, int concat_points) {
+                                double* tgrad_acc64, double* tgrad_abs64, float* ggs, double* ggs_abs64,
+                                int concat_points) {
     if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (double_backward<DD, float, double>(N, L, C, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, tgrad_acc64, tgrad_abs64, ggs, concat_points)));
+    DISPATCH_D(pos_dim, (double_backward<DD, float, double>(N, L, C, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, tgrad_acc64, tgrad_abs64, ggs, ggs_abs64, concat_points)));
     return 0;
 }
 
@@ -534,7 +578,7 @@ int penc_oracle_double_backward_f64(int pos_dim, int64_t N, int L, int C, const 
                                     const double* double_pos_grad, const double* grad, double* tgrad,
                                     double* ggs, int concat_points) {
     if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (double_backward<DD, double, double>(N, L, C, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, nullptr, nullptr, ggs, concat_points)));
+    DISPATCH_D(pos_dim, (double_backward<DD, double, double>(N, L, C, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, nullptr, nullptr, ggs, nullptr, concat_points)));
     return 0;
 }
 

@@ -44,8 +44,8 @@ _SIGNATURES = {
                                                            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_transpose": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
-                                          _c_f32p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, _c_f32p,
-                                          ctypes.c_void_p]),
+                                          _c_f32p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                          _c_f32p, ctypes.c_void_p]),
     "penc_probe_copy": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_void_p]),
     "penc_probe_gather": (ctypes.c_int, [_c_f32p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, _c_f32p,
                                          ctypes.c_void_p]),
@@ -304,8 +304,12 @@ class EncodingWrapper:
                 "double_backward_from_positions")
         return lv_grad, ggs
 
-    def simplex_debug(self, positions, capacity):
-        """Introspection: dict(rem0, rank, slot (int32), barycentric) each of shape (L, N, D+1)."""
+    def simplex_debug(self, positions, capacity, gather_path=False):
+        """Introspection: dict(rem0, rank, slot (int32), barycentric) each of shape (L, N, D+1).
+
+        ``gather_path`` picks the device routine whose slots and weights are reported: False for the
+        select chains of the scattering and position-gradient kernels, True for the LDS rank sort of
+        the forward and grad-of-grad kernels."""
         fp = self.fixed_params
         _check_f32_gpu(positions, "positions", 2)
         pos = positions.contiguous()
@@ -316,7 +320,8 @@ class EncodingWrapper:
         shift = fp.m_random_shift_per_level.contiguous()
         with torch.cuda.device(pos.device):
             _check(lib().penc_simplex_debug(self.pos_dim, n, levels, int(capacity), _ptr(pos),
-                                            _ptr(fp.m_scale_factor.to(pos.device)), _ptr(shift), _ptr(out["rem0"]),
+                                            _ptr(fp.m_scale_factor.to(pos.device)), _ptr(shift), int(bool(gather_path)),
+                                            _ptr(out["rem0"]),
                                             _ptr(out["rank"]), _ptr(out["slot"]), _ptr(out["barycentric"]), _stream()),
                    "simplex_debug")
         return out

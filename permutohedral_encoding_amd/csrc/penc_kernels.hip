@@ -315,7 +315,10 @@ grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mas
 // ------------------------------------------------------------------------------------------
 // introspection
 
-template <int D>
+// kViaLds selects which of the two equivalent device routines produce the slots and weights: the
+// compare-and-select chains (vertex_hashes / barycentric: table backward, position backward) or
+// the thread-private LDS column (sort_by_rank_lds: forward, grad-of-grad).
+template <int D, bool kViaLds>
 __global__ void __launch_bounds__(kBlock)
 simplex_debug_kernel(int n_points, uint32_t capacity, uint32_t cap_mask, const float* __restrict__ positions,
                      const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
@@ -325,8 +328,17 @@ simplex_debug_kernel(int n_points, uint32_t capacity, uint32_t cap_mask, const f
     if (n >= n_points) return;
     const int level = blockIdx.y;
     const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, scale_factor + level * D);
-    const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
-    const fvec<D + 1> w = barycentric<D>(s.rank, s.delta);
+    uvec<D + 1> h;
+    fvec<D + 1> w;
+    if constexpr (kViaLds) {
+        __shared__ uint2 columns[(D + 1) * kBlock];
+        fvec<D + 1> sorted;
+        sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, s.delta, s.hash0, sorted, h);
+        w = barycentric_of_sorted<D>(sorted);
+    } else {
+        h = vertex_hashes<D>(s.rank, s.hash0);
+        w = barycentric<D>(s.rank, s.delta);
+    }
     const size_t o = (static_cast<size_t>(level) * n_points + n) * (D + 1);
     static_for<D + 1>(PENC_BODY(i) {
         PENC_INDEX(i);
@@ -442,7 +454,7 @@ inline unsigned scatter_groups(int64_t n, int tiles_per_group) {
 // Tiles per scattering workgroup of the table backward.  Larger groups mean longer record segments
 // (less slack, longer bursts for the reducer) and fewer cache flushes; they are taken when the
 // launch still has several workgroups for every slot of the chip (measured: 3-13% faster then,
-// slower otherwise).  The double backward keeps kScatterTiles: it also gathers, a level at a time.
+// slower otherwise).  The same rule serves the scattering half of the double backward.
 inline int table_backward_tiles(int64_t n, int levels) {
     return static_cast<int64_t>(scatter_groups(n, kScatterTilesLarge)) * levels >= kLargeGroupsMinWorkgroups ? kScatterTilesLarge
                                                                                                             : kScatterTiles;
@@ -801,16 +813,23 @@ int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* s
 
 int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
                        const float* positions, const float* scale_factor, const float* random_shift,
-                       int* rem0, int* rank, int* slot, float* barycentric, void* stream) {
+                       int gather_path, int* rem0, int* rank, int* slot, float* barycentric, void* stream) {
     if (int rc = check_geometry(pos_dim, 2, nr_positions, nr_levels, capacity, 0)) return rc;
     if (nr_positions > ((int64_t{1} << 31) - 1) / (pos_dim + 1) / nr_levels) return PENC_ERR_BAD_SIZE;
     if (!positions || !scale_factor || !random_shift) return PENC_ERR_NULL_POINTER;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid(tiles(nr_positions), nr_levels);
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((simplex_debug_kernel<DD>), grid, dim3(kBlock), 0, st,
-                                                static_cast<int>(nr_positions), static_cast<uint32_t>(capacity),
-                                                mask_of(capacity), positions, scale_factor, random_shift, rem0, rank,
-                                                slot, barycentric));
+#define PENC_LAUNCH_DEBUG(VIA_LDS)                                                                                   \
+    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((simplex_debug_kernel<DD, VIA_LDS>), grid, dim3(kBlock), 0, st,       \
+                                                static_cast<int>(nr_positions), static_cast<uint32_t>(capacity),     \
+                                                mask_of(capacity), positions, scale_factor, random_shift, rem0, rank, \
+                                                slot, barycentric))
+    if (gather_path) {
+        PENC_LAUNCH_DEBUG(true);
+    } else {
+        PENC_LAUNCH_DEBUG(false);
+    }
+#undef PENC_LAUNCH_DEBUG
     return check_launch();
 }
 

@@ -18,6 +18,7 @@ orc = pytest.importorskip("oracle.api")
 DIMS = [2, 3, 4, 5, 6, 7, 8]
 FWD_RTOL, FWD_ATOL = 1e-5, 1e-6
 SUM_RTOL = 1e-4
+POS_RTOL = 1e-6  # sums of at most a few dozen levels, no atomics: far inside the 1e-4 bar
 
 
 def workload_problem(name, n):
@@ -33,7 +34,39 @@ def check_forward(got, want):
     assert np.all(err <= bound), f"forward: max err {err.max():.3g}, worst err/bound {np.max(err / bound):.3g}"
 
 
+def check_pos_grad(got, want):
+    """Position gradient against the oracle's fp64 sum of the same fp32 terms, per element, relative to
+    the chain of magnitudes behind that element (what its rounding error scales with).  The levels
+    are summed in a different but fixed order (pairs, then groups): observed worst case 8e-8."""
+    err = np.abs(got.astype(np.float64) - want["grad64"])
+    bound = POS_RTOL * want["abs64"] + 1e-30
+    assert np.all(err <= bound), f"position gradient: worst err/bound {np.max(err / bound):.3g} at rel {POS_RTOL}"
+
+
+def check_grad_grad(got, want):
+    """Gradient w.r.t. grad_sliced_values: the kernel performs the oracle's fp32 operations in the
+    oracle's order (no atomics are involved), so beyond the 1e-4 bar relative to the chain of
+    magnitudes it must be the same bits."""
+    err = np.abs(got.astype(np.float64) - want["ggs"].astype(np.float64))
+    bound = SUM_RTOL * want["ggs_abs64"] + 1e-30
+    assert np.all(err <= bound), f"grad-grad: worst err/bound {np.max(err / bound):.3g}"
+    assert np.array_equal(got, want["ggs"]), f"grad-grad: {np.mean(got != want['ggs']):.3g} of the values differ in the last bits"
+
+
 # ----------------------------------------------------------------------------- simplex, slots
+
+def check_simplex_bit_exact(enc, pos, want, capacity):
+    """rem0, rank, slots and weights of both device routines (select chains: scatter / position
+    kernels; LDS rank sort: forward / grad-of-grad kernels) against the oracle, bit for bit."""
+    pos_t = to_gpu(pos)
+    for gather_path in (False, True):
+        got = enc.simplex_debug(pos_t, capacity, gather_path=gather_path)
+        for k in ("rem0", "rank", "slot"):
+            assert np.array_equal(got[k].cpu().numpy(), want[k]), (k, gather_path)
+        # the weights are computed with the same operations in the same order
+        assert np.array_equal(got["barycentric"].cpu().numpy(), want["bary"]), gather_path
+        del got
+
 
 @pytest.mark.parametrize("d", DIMS)
 def test_simplex_rank_and_slots_bit_exact_all_dims(d):
@@ -43,11 +76,7 @@ def test_simplex_rank_and_slots_bit_exact_all_dims(d):
     want = orc.simplex(p["pos"], sf, p["shift"], cap)
     enc, fp = make_encoding(d, p["sigmas"], p["shift"])
     assert np.array_equal(fp.m_scale_factor.cpu().numpy(), sf)
-    got = enc.simplex_debug(to_gpu(p["pos"]), cap)
-    for k in ("rem0", "rank", "slot"):
-        assert np.array_equal(got[k].cpu().numpy(), want[k]), k
-    # the weights are computed with the same operations in the same order
-    assert np.array_equal(got["barycentric"].cpu().numpy(), want["bary"])
+    check_simplex_bit_exact(enc, p["pos"], want, cap)
 
 
 @pytest.mark.parametrize("name", ["c1", "c2", "c3", "c4", "c5"])
@@ -55,9 +84,29 @@ def test_simplex_bit_exact_on_benchmark_configs(name):
     w, p = workload_problem(name, 1 << 14)
     want = orc.simplex(p["pos"], p["sf"], p["shift"], w.capacity)
     enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
-    got = enc.simplex_debug(to_gpu(p["pos"]), w.capacity)
-    for k in ("rem0", "rank", "slot"):
-        assert np.array_equal(got[k].cpu().numpy(), want[k]), k
+    check_simplex_bit_exact(enc, p["pos"], want, w.capacity)
+
+
+@pytest.mark.parametrize("d", DIMS)
+def test_rounding_ties_and_lattice_points_bit_exact(d):
+    """Points whose elevated coordinates sit exactly on rounding ties, on lattice points and on
+    simplex faces (unit scale factors, no shift, coordinates that are multiples of 1/4): the two
+    hand-worked tie cases of the oracle's pinning tests, then a grid of them against the oracle."""
+    from test_oracle_pinning import TIE_CASES
+    enc, fp = make_encoding(d, np.ones(1, np.float32), np.zeros((1, d), np.float32))
+    fp.m_scale_factor = torch.ones((1, d), device="cuda")
+    for dd, pos, _, rem0, rank, bary in TIE_CASES:
+        if dd == d:
+            for gather_path in (False, True):
+                got = enc.simplex_debug(to_gpu(np.array([pos], np.float32)), 1 << 16, gather_path=gather_path)
+                assert got["rem0"][0, 0].tolist() == rem0 and got["rank"][0, 0].tolist() == rank
+                assert got["barycentric"][0, 0].tolist() == bary
+    rng = np.random.default_rng(d)
+    pos = (rng.integers(-40, 41, size=(20000, d)) * 0.25).astype(np.float32)
+    pos[:200, 1:] = 0.0
+    pos[:200, 0] = (np.arange(200) - 100) * 0.25 * (d + 1)  # walks through every tie of the first two coordinates
+    want = orc.simplex(pos, np.ones((1, d), np.float32), np.zeros((1, d), np.float32), 1 << 16)
+    check_simplex_bit_exact(enc, pos, want, 1 << 16)
 
 
 # ----------------------------------------------------------------------------- the five configs, reduced N
@@ -78,17 +127,13 @@ def test_config_all_phases_match_oracle(name):
     want = orc.backward_table(p["pos"], p["sf"], p["shift"], p["window"], p["grad"], w.capacity, want32=False, want_abs=True)
     assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
     del want
-    wantp = orc.backward_pos(p["pos"], p["table"], p["sf"], p["shift"], p["window"], p["grad"])["grad64"]
-    scale = np.abs(wantp).max(axis=1, keepdims=True)
-    assert np.all(np.abs(pg.cpu().numpy() - wantp) <= SUM_RTOL * (np.abs(wantp) + scale) + 1e-30)
+    check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], p["sf"], p["shift"], p["window"], p["grad"]))
 
     tg2, ggs = enc.double_backward_from_positions(inp, dpos_t, grad_t)
     want = orc.double_backward(p["pos"], p["table"], p["sf"], p["shift"], p["window"], p["dpos"], p["grad"],
                                want32=False, want_abs=True)
     assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient")
-    ggs = ggs.cpu().numpy()
-    lvl_scale = np.abs(want["ggs"]).max(axis=(1, 2), keepdims=True)
-    assert np.all(np.abs(ggs - want["ggs"]) <= SUM_RTOL * (np.abs(want["ggs"]) + lvl_scale) + 1e-30)
+    check_grad_grad(ggs.cpu().numpy(), want)
 
 
 @pytest.mark.parametrize("d", DIMS)
@@ -102,14 +147,11 @@ def test_all_dims_all_phases_match_oracle(d):
     tg, pg = enc.backward(inp, to_gpu(p["grad"]))
     want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
     assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
-    wantp = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])["grad64"]
-    scale = np.abs(wantp).max(axis=1, keepdims=True)
-    assert np.all(np.abs(pg.cpu().numpy() - wantp) <= SUM_RTOL * (np.abs(wantp) + scale))
+    check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"]))
     tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
     want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
     assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient")
-    lvl_scale = np.abs(want["ggs"]).max(axis=(1, 2), keepdims=True)
-    assert np.all(np.abs(ggs.cpu().numpy() - want["ggs"]) <= SUM_RTOL * (np.abs(want["ggs"]) + lvl_scale))
+    check_grad_grad(ggs.cpu().numpy(), want)
 
 
 # ----------------------------------------------------------------------------- edge cases
@@ -177,8 +219,7 @@ def test_masked_levels_are_exact_zeros_and_noops():
     assert torch.all(tg[3:] == 0) and not torch.all(tg[:3] == 0)
     tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
     assert torch.all(tg2[3:] == 0) and torch.all(ggs[3:] == 0)
-    wantp = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])["grad64"]
-    assert np.allclose(pg.cpu().numpy(), wantp, rtol=1e-4, atol=1e-4 * np.abs(wantp).max())
+    check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"]))
 
 
 def test_only_one_gradient_requested():
@@ -223,12 +264,67 @@ def test_error_paths():
     assert torch.equal(out, enc.forward(good))
 
 
+# ----------------------------------------------------------------------------- the five configs at their stated sizes
+
+FULL_SIZE_PHASES = [(name, phase) for name in ("c1", "c2", "c3", "c4", "c5")
+                    for phase in ("simplex",) + wl.WORKLOADS[name].phases]
+
+
+@pytest.mark.parametrize("name,phase", FULL_SIZE_PHASES, ids=[f"{n}-{ph}" for n, ph in FULL_SIZE_PHASES])
+def test_full_size_config_matches_oracle(name, phase):
+    """Every phase a benchmark configuration names, at the configuration's own size (2^16 points for
+    c1, 2^19 for c4, 2^20 otherwise), against the oracle on all points, levels and slots: the large
+    point groups, the level interleave over the dies, the bins of a 2^22-slot table and the
+    multi-workgroup bin reducer are only in use at these sizes."""
+    w = wl.WORKLOADS[name]
+    need = {"simplex": ("shift", "pos"), "forward": ("table", "shift", "pos"),
+            "backward_table": ("shift", "pos", "grad"), "backward_pos": ("table", "shift", "pos", "grad"),
+            "double_backward": ("table", "shift", "pos", "grad", "dpos")}[phase]
+    p = wl.make_inputs(w, need=need)
+    sf = orc.scale_factors(w.pos_dim, p["sigmas"])
+    enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
+    from permutohedral_encoding_amd import _native
+
+    if phase == "simplex":  # in slabs of points: (L, N, D+1) int32 arrays of the oracle and of both device routines
+        slab = 1 << 17
+        for first in range(0, w.nr_points, slab):
+            pos = p["pos"][first:first + slab]
+            check_simplex_bit_exact(enc, pos, orc.simplex(pos, sf, p["shift"], w.capacity), w.capacity)
+        return
+
+    pos_t, win_t = to_gpu(p["pos"]), to_gpu(p["window"])
+    table_t = to_gpu(p["table"]) if "table" in p else torch.zeros((w.nr_levels, 1, 2), device="cuda")
+    if phase == "forward":
+        out = enc.forward(_native.EncodingInput(table_t, pos_t, win_t, False, False)).cpu().numpy()
+        want = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"])
+        check_forward(out, want)
+        assert np.array_equal(out, want), "same fp32 operations in the same order: the bits must agree"
+        if w.masked_top_levels:
+            assert np.all(out[w.nr_levels - w.masked_top_levels:] == 0.0)
+    elif phase == "backward_table":
+        table_t = torch.zeros((w.nr_levels, w.capacity, 2), device="cuda")  # never read by the table gradient
+        tg, _ = enc.backward(_native.EncodingInput(table_t, pos_t, win_t, True, False), to_gpu(p["grad"]))
+        want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], w.capacity, want32=False, want_abs=True)
+        assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+        if w.masked_top_levels:
+            assert torch.all(tg[w.nr_levels - w.masked_top_levels:] == 0.0)
+    elif phase == "backward_pos":
+        _, pg = enc.backward(_native.EncodingInput(table_t, pos_t, win_t, False, True), to_gpu(p["grad"]))
+        check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"]))
+    else:
+        tg2, ggs = enc.double_backward_from_positions(_native.EncodingInput(table_t, pos_t, win_t, True, True),
+                                                      to_gpu(p["dpos"]), to_gpu(p["grad"]))
+        want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"],
+                                   want32=False, want_abs=True)
+        assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient")
+        check_grad_grad(ggs.cpu().numpy(), want)
+
+
 # ----------------------------------------------------------------------------- size-independent properties at full size
 
 @pytest.mark.parametrize("name", ["c2", "c3", "c4", "c5"])
 def test_full_size_adjoint_identities(name):
-    """forward is linear in the table and the position gradient bilinear in (table, grad): at the
-    full benchmark sizes, where the CPU oracle would take minutes,
+    """forward is linear in the table and the position gradient bilinear in (table, grad), so at any size
         <forward(T), g> = <T, table_grad(g)>
         <q, pos_grad(T, g)> = <ggs(q, T), g> = <table_grad2(q, g), T>
     must hold (fp64 dot products of the fp32 results)."""
@@ -356,8 +452,7 @@ def test_position_gradient_with_and_without_workspace():
     p = random_problem(d, 5000, 7, cap, seed=12, sigma_range=(1.0, 1e-3))  # 7 levels: a ragged last group
     sf = orc.scale_factors(d, p["sigmas"])
     enc, _ = make_encoding(d, p["sigmas"], p["shift"])
-    want = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])["grad64"]
-    scale = np.abs(want).max(axis=1, keepdims=True)
+    want = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])
     results = []
     for lpp in (0, -1, 0):
         _native.LEVELS_PER_PASS = lpp
@@ -366,7 +461,7 @@ def test_position_gradient_with_and_without_workspace():
         finally:
             _native.LEVELS_PER_PASS = 0
         got = pg.cpu().numpy()
-        assert np.all(np.abs(got - want) <= SUM_RTOL * (np.abs(want) + scale))
+        check_pos_grad(got, want)
         results.append(got)
     assert np.array_equal(results[0], results[2])
 

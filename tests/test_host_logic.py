@@ -59,7 +59,9 @@ def test_argument_validation_without_a_gpu():
     assert lib.penc_backward(3, 2, 10, 2, 16, p, p, p, p, p, p, z, z, None, 0, None) == 1
     assert lib.penc_backward(3, 2, 10, 2, 16, p, z, p, p, p, p, z, p, None, 0, None) == 1
     assert lib.penc_double_backward_from_positions(3, 2, 10, 2, 16, p, p, p, p, p, p, p, z, z, 0, None, 0, None) == 1
-    assert lib.penc_simplex_debug(3, 0, 2, 16, p, p, p, z, z, z, z, None) == 2
+    assert lib.penc_simplex_debug(3, 0, 2, 16, p, p, p, 0, z, z, z, z, None) == 2
+    assert lib.penc_backward_static(3, 2, 0, 2, 16, p, p, p, p, p, p, p, z, None) == 2
+    assert lib.penc_backward_static(3, 2, 1 << 24, 2, 1 << 18, p, p, p, p, p, p, p, z, None) == 7  # before any pointer is read
     assert lib.penc_scale_factors(3, 2, z, p) == 1
     # workspace sizing: grows with the levels per pass, 0 when the capacity cannot be binned
     w1 = lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 1)

@@ -196,6 +196,37 @@ def test_simplex_hand_case_2d():
     assert s["slot"][0, 0].tolist() == [0, poly_hash((1, -2)) % (1 << 16), poly_hash((2, -1)) % (1 << 16)]
 
 
+# Rounding ties.  A coordinate of the elevated point exactly halfway between two multiples of D+1
+# takes the lower one (the comparison `up - e < e - down` is strict, EncodingGPU.cuh:153-157).
+# Worked by hand, D = 3, pos = (2, 0, 0), unit scale factors, no shift:
+#   elevated = (2, -2, 0, 0); both 2 and -2 are ties: rounded down to 0 and -4; sum/4 = -1
+#   residuals (2, 2, 0, 0) -> ranks (0, 1, 2, 3) (equal residuals: the lower index ranks first), plus
+#   the sum: (-1, 0, 1, 2); rank 0 wraps to 3 and its rem0 to 4  =>  rem0 (4, -4, 0, 0), rank (3, 0, 1, 2)
+#   delta = (elevated - rem0)/4 = (-1/2, 1/2, 0, 0)  =>  weights (0, 1/2, 0, 1/2)
+# and D = 2, pos = (1.5, 0): elevated (1.5, -1.5, 0) -> rem0 (3, -3, 0), rank (2, 0, 1), weights (0, 1/2, 1/2).
+# (Taking the upper multiple at a tie instead ends in the same rem0, rank and weights: the tied
+# coordinates then have the smallest residuals instead of the largest, the sum is larger by their
+# number, and the wrap puts them back in front in index order.  So the direction of the tie is
+# not observable, which the mutation check of these tests confirms; the values below are.)
+TIE_CASES = [
+    (3, [2.0, 0.0, 0.0], [2.0, -2.0, 0.0, 0.0], [4, -4, 0, 0], [3, 0, 1, 2], [0.0, 0.5, 0.0, 0.5]),
+    (2, [1.5, 0.0], [1.5, -1.5, 0.0], [3, -3, 0], [2, 0, 1], [0.0, 0.5, 0.5]),
+]
+
+
+@pytest.mark.parametrize("d,pos,elevated,rem0,rank,bary", TIE_CASES)
+def test_rounding_tie_hand_worked(d, pos, elevated, rem0, rank, bary):
+    s = orc.simplex(np.array([pos], np.float32), np.ones((1, d), np.float32), np.zeros((1, d), np.float32), 1 << 16,
+                    with_keys=True)
+    assert s["elevated"][0, 0].tolist() == elevated
+    assert s["rem0"][0, 0].tolist() == rem0
+    assert s["rank"][0, 0].tolist() == rank
+    assert s["bary"][0, 0].tolist() == bary
+    keys = [[rem0[i] + r - (d + 1) * (rank[i] > d - r) for i in range(d + 1)] for r in range(d + 1)]
+    assert s["keys"][0, 0].tolist() == keys
+    assert s["slot"][0, 0].tolist() == [poly_hash(k[:d]) % (1 << 16) for k in keys]
+
+
 # ----------------------------------------------------------------------------- forward
 
 def _collision_free(d, dtype, n=512, levels=4, seed=1, capacity=1 << 22):
