@@ -58,8 +58,9 @@ const char* penc_status_string(int status);
  * Replaces: src/Encoding.cu:71-74 and src/pytorch_modules/modules.py:95-103. */
 int penc_extra_levels(int pos_dim, int nr_feat, int concat_points);
 
-/* scale_factor_out[l][i] = fp32(1/sqrt((i+1)(i+2))) / sigmas[l], a true fp32 division.
- * Both arrays are HOST memory.
+/* scale_factor_out[l][i] = fp32(1/sqrt((i+1)(i+2))) * (1.0f / sigmas[l]): the fp32 result of the
+ * reference's "tensor element / host scalar", which ATen evaluates as a multiplication by the
+ * rounded reciprocal.  Both arrays are HOST memory.
  * Replaces: EncodingFixedParams::compute_scale_factor_tensor, Encoding.cuh:55-69. */
 int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* scale_factor_out);
 

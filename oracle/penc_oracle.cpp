@@ -449,14 +449,18 @@ void double_backward(int64_t N, int L, int C, const R* pos, const R* table, cons
 }
 
 // include/permutohedral_encoding/Encoding.cuh:55-69.  The numerator is evaluated in fp64 and
-// rounded to fp32 when stored, then divided by the fp32 sigma.  The rule fixed here (and in the
-// shipped library) is a true fp32 division.
-// Pinned by: closed form 1/(sqrt((i+1)(i+2)) * sigma) within 1.5 ulp (two fp32 roundings).
+// rounded to fp32 when it is stored in the tensor (":62"); the division of that fp32 tensor element
+// by the fp32 sigma (":63") is ATen's tensor / host-scalar, which multiplies by the rounded fp32
+// reciprocal of the scalar (its "a * (1/b)" path for a scalar second operand).
+// Pinned by: closed form 1/(sqrt((i+1)(i+2)) * sigma) within 2 ulp (three fp32 roundings); the choice
+// between this rule and a true division (1 ulp apart for a quarter of the entries) by a GPU test
+// that evaluates the reference's two statements with torch itself.
 void scale_factors(int D, int L, const float* sigmas, float* sf) {
     for (int l = 0; l < L; ++l)
         for (int i = 0; i < D; ++i) {
             const float num = static_cast<float>(1.0 / std::sqrt(static_cast<double>((i + 1) * (i + 2))));
-            sf[l * D + i] = num / sigmas[l];
+            const float reciprocal = 1.0f / sigmas[l];
+            sf[l * D + i] = num * reciprocal;
         }
 }
 

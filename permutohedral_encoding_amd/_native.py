@@ -14,7 +14,8 @@ import numpy as np
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libpenc_hip.so")
+# PENC_HIP_LIB names another build of the same library (kernel experiments, a debug build)
+LIB_PATH = os.environ.get("PENC_HIP_LIB", os.path.join(_HERE, "libpenc_hip.so"))
 _lib = None
 
 _c_f32p = ctypes.c_void_p

@@ -492,9 +492,10 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int t
         if (bytes < segments * (sizeof(uint32_t) + 16 * sizeof(BinRecord))) return p;
         cap = static_cast<uint32_t>((bytes / segments - sizeof(uint32_t)) / sizeof(BinRecord));
     }
-    // the scattering kernel indexes a level's records with 32 bits
-    if (segments * cap > 0xFFFFFFFFull) {
-        cap = static_cast<uint32_t>(0xFFFFFFFFull / segments);
+    // the scattering kernel addresses a level's records with 32-bit byte offsets
+    constexpr uint64_t kMaxRecordsPerLevel = 0xFFFFFFFFull / sizeof(BinRecord);
+    if (segments * cap > kMaxRecordsPerLevel) {
+        cap = static_cast<uint32_t>(kMaxRecordsPerLevel / segments);
         if (cap < 16) return p;
     }
     const size_t fit = bytes / bin_bytes_per_level(n_bins, n_groups, cap);
@@ -700,8 +701,12 @@ int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* s
     if (pos_dim < 1 || nr_levels < 1) return PENC_ERR_BAD_SIZE;
     for (int l = 0; l < nr_levels; ++l)
         for (int i = 0; i < pos_dim; ++i) {
+            // the reference divides a float32 tensor element by a host scalar (Encoding.cuh:62-63), which ATen
+            // evaluates as element * (1.0f / scalar): two roundings, up to one unit in the last place away
+            // from a true division
             const float numerator = static_cast<float>(1.0 / __builtin_sqrt(static_cast<double>((i + 1) * (i + 2))));
-            scale_factor_out[l * pos_dim + i] = numerator / sigmas[l];
+            const float reciprocal = 1.0f / sigmas[l];
+            scale_factor_out[l * pos_dim + i] = numerator * reciprocal;
         }
     return PENC_OK;
 }

@@ -228,7 +228,11 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
 // its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
-// Needs bins.n_bins <= kStageBins and a level's record array below 2^32 records (the host plans
+// A staged record carries its destination (byte offset / 12 in the level's record array), so the
+// store needs no search.  When a run does not fit its segment any more (rare: the segments hold
+// the mean plus three standard deviations) the whole chunk takes the careful path, which checks
+// every record against the room left and sends the excess to stage 3.
+// Needs bins.n_bins <= kStageBins and a level's record array below 2^32 bytes (the host plans
 // for both); all 64 lanes of the wave must call it together.
 template <int D>
 __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
@@ -245,6 +249,7 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
     uint32_t* start = count + 128;  // index of the run's first record in the level's record array
     uint32_t* room = count + 192;   // records the workgroup's segment of the bin can still take
     uint4* stage = reinterpret_cast<uint4*>(c.val) + wave * (kStageChunk * 64);
+    char* const record_bytes = reinterpret_cast<char*>(bins.records);
     constexpr uint32_t kNoRoom = 0xFFFFFFFFu;
     constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
     static_for<kChunks>(PENC_BODY(chunk) {
@@ -265,43 +270,74 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
         offset[lane] = wave_exclusive_scan(mine, total);
         const uint32_t taken = mine != 0u ? atomicAdd(&c.bin_count[lane], mine) : 0u;
         start[lane] = (lane * bins.n_groups + group) * bins.segment_capacity + taken;
-        room[lane] = taken < bins.segment_capacity ? bins.segment_capacity - taken : 0u;
-        wave_lds_fence();
-        static_for<kCount>(PENC_BODY(j) {
-            PENC_INDEX(j);
-            if (active) {
-                const uint32_t b = slot[kFirst + j] >> kBinSlotsLog2;
-                // copies first: a bit cast applied directly to a vector element reads element 0
-                const float v0 = a0[kFirst + j], v1 = a1[kFirst + j];
-                uint4 e;
-                e.x = slot[kFirst + j];
-                e.y = __builtin_bit_cast(uint32_t, v0);
-                e.z = __builtin_bit_cast(uint32_t, v1);
-                e.w = place[j] < room[b] ? start[b] + place[j] : kNoRoom;
-                stage[offset[b] + place[j]] = e;
-            }
-        });
-        wave_lds_fence();
-        static_for<kCount>(PENC_BODY(j) {
-            PENC_INDEX(j);
-            const uint32_t i = j * 64 + lane;
-            bool spill = false;
-            uint4 e = {0u, 0u, 0u, 0u};
-            if (i < total) {
-                e = stage[i];
-                if (e.w != kNoRoom) {
+        const bool fits = taken + mine <= bins.segment_capacity;
+        if (__all(fits)) {
+            wave_lds_fence();
+            static_for<kCount>(PENC_BODY(j) {
+                PENC_INDEX(j);
+                if (active) {
+                    const uint32_t b = slot[kFirst + j] >> kBinSlotsLog2;
+                    // copies first: a bit cast applied directly to a vector element reads element 0
+                    const float v0 = a0[kFirst + j], v1 = a1[kFirst + j];
+                    uint4 e;
+                    e.x = slot[kFirst + j] & (kBinSlots - 1);
+                    e.y = __builtin_bit_cast(uint32_t, v0);
+                    e.z = __builtin_bit_cast(uint32_t, v1);
+                    e.w = start[b] + place[j];
+                    stage[offset[b] + place[j]] = e;
+                }
+            });
+            wave_lds_fence();
+            static_for<kCount>(PENC_BODY(j) {
+                PENC_INDEX(j);
+                const uint32_t i = j * 64 + lane;
+                if (i < total) {
+                    const uint4 e = stage[i];
                     BinRecord rec;
-                    rec.slot_in_bin = e.x & (kBinSlots - 1);
+                    rec.slot_in_bin = e.x;
                     rec.a0 = __builtin_bit_cast(float, e.y);
                     rec.a1 = __builtin_bit_cast(float, e.z);
-                    bins.records[e.w] = rec;
-                } else {
-                    spill = true;  // the segment is full: stage 3
+                    *reinterpret_cast<BinRecord*>(record_bytes + e.w * static_cast<uint32_t>(sizeof(BinRecord))) = rec;
                 }
-            }
-            if (__any(spill))
-                global_add_pairs(level_grad, spill, e.x, __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
-        });
+            });
+        } else {
+            room[lane] = taken < bins.segment_capacity ? bins.segment_capacity - taken : 0u;
+            wave_lds_fence();
+            static_for<kCount>(PENC_BODY(j) {
+                PENC_INDEX(j);
+                if (active) {
+                    const uint32_t b = slot[kFirst + j] >> kBinSlotsLog2;
+                    const float v0 = a0[kFirst + j], v1 = a1[kFirst + j];
+                    uint4 e;
+                    e.x = slot[kFirst + j];
+                    e.y = __builtin_bit_cast(uint32_t, v0);
+                    e.z = __builtin_bit_cast(uint32_t, v1);
+                    e.w = place[j] < room[b] ? start[b] + place[j] : kNoRoom;
+                    stage[offset[b] + place[j]] = e;
+                }
+            });
+            wave_lds_fence();
+            static_for<kCount>(PENC_BODY(j) {
+                PENC_INDEX(j);
+                const uint32_t i = j * 64 + lane;
+                bool spill = false;
+                uint4 e = {0u, 0u, 0u, 0u};
+                if (i < total) {
+                    e = stage[i];
+                    if (e.w != kNoRoom) {
+                        BinRecord rec;
+                        rec.slot_in_bin = e.x & (kBinSlots - 1);
+                        rec.a0 = __builtin_bit_cast(float, e.y);
+                        rec.a1 = __builtin_bit_cast(float, e.z);
+                        bins.records[e.w] = rec;
+                    } else {
+                        spill = true;  // the segment is full: stage 3
+                    }
+                }
+                if (__any(spill))
+                    global_add_pairs(level_grad, spill, e.x, __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
+            });
+        }
         wave_lds_fence();
     });
 }
@@ -432,7 +468,10 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
 __global__ void __launch_bounds__(kReduceBlock)
 bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity,
                   float* __restrict__ table_grad, int first_level) {
-    __shared__ double acc[kBinSlots][2];
+    // one array per feature: lanes that hit different slots then spread over all bank pairs (interleaved
+    // features would leave every other pair idle in each of the two adds)
+    __shared__ double acc0[kBinSlots];
+    __shared__ double acc1[kBinSlots];
     const uint32_t bin = blockIdx.x;
     // last level first: with the usual coarse-to-fine level list the bins with the most records are
     // started first and the nearly empty ones fill the tail of the launch
@@ -441,8 +480,8 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
-        acc[s][0] = 0.0;
-        acc[s][1] = 0.0;
+        acc0[s] = 0.0;
+        acc1[s] = 0.0;
     }
     __syncthreads();
     constexpr uint32_t kWaves = kReduceBlock / 64;
@@ -487,9 +526,9 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
 #pragma unroll
             for (uint32_t u = 0; u < kUnroll; ++u)
                 if (base + u * 64 + lane < count) {
-                    double* cell = acc[cur[u].slot_in_bin];
-                    __hip_atomic_fetch_add(cell, static_cast<double>(cur[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(cell + 1, static_cast<double>(cur[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    const uint32_t cell = cur[u].slot_in_bin;
+                    __hip_atomic_fetch_add(&acc0[cell], static_cast<double>(cur[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&acc1[cell], static_cast<double>(cur[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 }
 #pragma unroll
             for (uint32_t u = 0; u < kUnroll; ++u) cur[u] = next[u];
@@ -502,7 +541,7 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     const uint32_t slot0 = bin << kBinSlotsLog2;
     const bool alone = gridDim.z == 1;
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
-        const double v0 = acc[s][0], v1 = acc[s][1];
+        const double v0 = acc0[s], v1 = acc1[s];
         if ((v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity) {
             if (alone) {
                 float2 g = level_grad[slot0 + s];

@@ -55,6 +55,26 @@ def check_grad_grad(got, want):
 
 # ----------------------------------------------------------------------------- simplex, slots
 
+@pytest.mark.parametrize("name", ["c2", "c3", "c4"])
+def test_scale_factors_follow_torch_division_by_a_host_scalar(name):
+    """The reference fills its scale-factor tensor with `t[l][i] = 1/sqrt((i+1)(i+2))` followed by
+    `t[l][i] = t[l][i] / sigma_l` on a float32 GPU tensor (Encoding.cuh:62-63).  Those two statements,
+    evaluated by torch itself on this GPU, must give the bits penc_scale_factors computes on the host
+    (torch multiplies by the rounded reciprocal of a host scalar; a true division differs by one
+    unit in the last place for about a quarter of the entries)."""
+    from permutohedral_encoding_amd import _native
+    w = wl.WORKLOADS[name]
+    sig = wl.scale_list(w)
+    t = torch.zeros((w.nr_levels, w.pos_dim), dtype=torch.float32, device="cuda")
+    for l in range(w.nr_levels):
+        for i in range(w.pos_dim):
+            t[l][i] = 1.0 / np.sqrt(float((i + 1) * (i + 2)))
+            t[l][i] = t[l][i] / float(sig[l])
+    got = _native.scale_factors(w.pos_dim, sig)
+    assert np.array_equal(got, t.cpu().numpy())
+    assert np.array_equal(got, orc.scale_factors(w.pos_dim, sig))
+
+
 def check_simplex_bit_exact(enc, pos, want, capacity):
     """rem0, rank, slots and weights of both device routines (select chains: scatter / position
     kernels; LDS rank sort: forward / grad-of-grad kernels) against the oracle, bit for bit."""

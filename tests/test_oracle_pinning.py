@@ -5,7 +5,7 @@ is pinned by a closed form, an invariant or a brute-force property chosen so tha
 mistake (a dropped term, a wrong sign or index, a transposed operand) fails:
 
   hash                  known answers evaluated as a polynomial in Python integers
-  scale factors         closed form within 1.5 ulp (two fp32 roundings)
+  scale factors         closed form within 2 ulp (three fp32 roundings); division rule by a GPU test against torch
   elevation             sum = 0 and |E| = |pos+shift|/sigma (scaled isometry)
   simplex / rank / keys vertices are A_d* lattice points forming a canonical simplex that
                         contains the point: sum_r b_r * vertex_r = E, b >= 0, sum b = 1
@@ -80,8 +80,11 @@ def test_scale_factors_closed_form(d):
     i = np.arange(d, dtype=np.float64)
     want = 1.0 / (np.sqrt((i + 1) * (i + 2))[None, :] * sig.astype(np.float64)[:, None])
     ulp = np.spacing(want.astype(np.float32)).astype(np.float64)
-    # two fp32 roundings (the numerator, then the quotient): at most 0.5 + 1 ulp from the exact value
-    assert np.all(np.abs(sf.astype(np.float64) - want) <= 1.5 * ulp)
+    # three fp32 roundings (the numerator, the reciprocal of sigma, their product): at most 2 ulp from the exact value
+    assert np.all(np.abs(sf.astype(np.float64) - want) <= 2.0 * ulp)
+    # and exactly the rule fp32(numerator) * fp32(1 / sigma)
+    num = (1.0 / np.sqrt((i + 1) * (i + 2))).astype(np.float32)
+    assert np.array_equal(sf, num[None, :] * (np.float32(1.0) / sig)[:, None])
 
 
 # ----------------------------------------------------------------------------- elevation + simplex
