@@ -154,27 +154,41 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
     scatter_begin(state);
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
-    const auto load_grad = [&](int n, float& g0, float& g1) {
+    // Everything a thread reads lies within its group of at most 16 x 512 points, so the addresses are
+    // wave-uniform 64-bit bases (scalar registers) plus 32-bit per-thread offsets.
+    const uint32_t last_in_group = static_cast<uint32_t>(n_points - 1 - group_base);
+    const float* const group_positions = positions + group_base * D;
+    const float* const group_q = kSecondOrder ? double_pos_grad + group_base * D : nullptr;
+    const float* const group_grad0 =
+        kRowMajor ? grad_sliced + group_base * grad_row_stride + 2 * level
+                  : grad_sliced + (static_cast<size_t>(level) * 2) * n_points + group_base;
+    const float* const group_grad1 = group_grad0 + n_points;
+    const auto load_grad = [&](uint32_t i, float& g0, float& g1) {
         if constexpr (kRowMajor) {
-            const float2 g = *reinterpret_cast<const float2*>(grad_sliced + static_cast<int64_t>(n) * grad_row_stride + 2 * level);
+            const float2 g = *reinterpret_cast<const float2*>(group_grad0 + static_cast<int64_t>(i) * grad_row_stride);
             g0 = g.x;
             g1 = g.y;
         } else {
-            const float* g0p = grad_sliced + (static_cast<size_t>(level) * 2) * n_points;
-            g0 = g0p[n];
-            g1 = g0p[static_cast<size_t>(n_points) + n];
+            g0 = group_grad0[i];
+            g1 = group_grad1[i];
         }
+    };
+    const auto load_group_point = [&](const float* base, uint32_t i) {
+        fvec<D> v;
+        static_for<D>(PENC_BODY(k) {
+            PENC_INDEX(k); v[k] = base[i * static_cast<uint32_t>(D) + k]; });
+        return v;
     };
     // A tile's inputs are fetched one tile ahead: their latency then overlaps the previous tile's
     // scatter instead of stalling the wave at the top of every iteration.
-    const auto point_of = [&](int t) {  // the point this thread handles in tile t (clamped: the tail re-reads the last point)
-        const int64_t n = group_base + static_cast<int64_t>(t) * kScatterBlock + threadIdx.x;
-        return static_cast<int>(n < n_points ? n : n_points - 1);
+    const auto point_of = [&](int t) {  // the point this thread handles in tile t, within the group (clamped: the tail re-reads the last point)
+        const uint32_t i = static_cast<uint32_t>(t) * kScatterBlock + threadIdx.x;
+        return i < last_in_group ? i : last_in_group;
     };
-    int nn = point_of(0);
-    fvec<D> pos = load_point<D>(positions, nn);
+    uint32_t nn = point_of(0);
+    fvec<D> pos = load_group_point(group_positions, nn);
     fvec<D> q = 0.0f;
-    if constexpr (kSecondOrder) q = load_point<D>(double_pos_grad, nn);
+    if constexpr (kSecondOrder) q = load_group_point(group_q, nn);
     float g0, g1;
     load_grad(nn, g0, g1);
     bool streaming = false;
@@ -182,10 +196,10 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
         const int64_t tile_base = group_base + static_cast<int64_t>(t) * kScatterBlock;
         if (tile_base >= n_points) break;
         const bool active = tile_base + threadIdx.x < n_points;
-        const int nn_next = point_of(t + 1);
-        const fvec<D> pos_next = load_point<D>(positions, nn_next);
+        const uint32_t nn_next = point_of(t + 1);
+        const fvec<D> pos_next = load_group_point(group_positions, nn_next);
         fvec<D> q_next = 0.0f;
-        if constexpr (kSecondOrder) q_next = load_point<D>(double_pos_grad, nn_next);
+        if constexpr (kSecondOrder) q_next = load_group_point(group_q, nn_next);
         float g0_next, g1_next;
         load_grad(nn_next, g0_next, g1_next);
         if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);

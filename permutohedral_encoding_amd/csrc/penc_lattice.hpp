@@ -115,18 +115,18 @@ __device__ __forceinline__ Located<D> locate(fvec<D> pos, const float* __restric
     });
     elevated[0] = sm;
 
-    fvec<D1> base;   // the chosen multiple of D+1 as a float (exact)
-    fvec<D1> resid;
+    // Round every coordinate to the nearer multiple of D+1, the lower one at a tie (:149-158).  The
+    // upper candidate is formed as down + (D+1) instead of ceil(v)*(D+1): the two differ only when v
+    // is an integer, where the reference's candidates coincide and the lower one is chosen here too.
+    fvec<D1> resid;  // elevated - rounded: exact in fp32 (the two are within (D+1)/2 of each other)
     ivec<D1> rem0;
     int sum = 0;
     static_for<D1>(PENC_BODY(i) {
         PENC_INDEX(i);
         const float e = elevated[i];
-        const float v = e * kInv;
-        const float up = __builtin_ceilf(v) * static_cast<float>(D1);
-        const float down = __builtin_floorf(v) * static_cast<float>(D1);
+        const float down = __builtin_floorf(e * kInv) * static_cast<float>(D1);
+        const float up = down + static_cast<float>(D1);
         const float b = (up - e < e - down) ? up : down;
-        base[i] = b;
         rem0[i] = static_cast<int>(b);
         resid[i] = e - b;
         sum += static_cast<int>(b);
@@ -145,17 +145,26 @@ __device__ __forceinline__ Located<D> locate(fvec<D> pos, const float* __restric
         });
     });
 
+    // Wrap back onto the hyperplane (:173-186): a rank pushed outside 0..D by the coordinate sum comes
+    // back by D+1 and takes its rem0 along.  `moved` is that multiple of D+1 (0 or +-(D+1)).  The
+    // residual after the wrap, elevated - (rounded + moved), is one rounding of an exact difference
+    // whichever way it is bracketed, so it is formed from the (exact) residual before the wrap.
     Located<D> o;
     uint32_t h = 0u;
     static_for<D1>(PENC_BODY(i) {
         PENC_INDEX(i);
         const int rk = rank[i] + sum;
-        const int wrap = rk < 0 ? 1 : (rk > D ? -1 : 0);
-        o.rank[i] = rk + wrap * D1;
-        const int r0 = rem0[i] + wrap * D1;
+        int wrapped_rank;
+        if constexpr ((D1 & (D1 - 1)) == 0) {
+            wrapped_rank = rk & (D1 - 1);  // rk is within D+1 of 0..D: reduction modulo a power of two
+        } else {
+            wrapped_rank = rk < 0 ? rk + D1 : (rk > D ? rk - D1 : rk);
+        }
+        const int moved = wrapped_rank - rk;
+        o.rank[i] = wrapped_rank;
+        const int r0 = rem0[i] + moved;
         o.rem0[i] = r0;
-        const float wrapped = base[i] + static_cast<float>(wrap * D1);
-        o.delta[i] = (elevated[i] - wrapped) * kInv;
+        o.delta[i] = (resid[i] - static_cast<float>(moved)) * kInv;
         if constexpr (i < D) h += static_cast<uint32_t>(r0) * hash_pow(D - i);
     });
     o.hash0 = h;

@@ -163,7 +163,7 @@ __device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad,
 // slow on this chip.  The fp64 partial sums are rounded to fp32 once, when the cache is flushed.
 struct ScatterState {
     int tag[kCacheLines];
-    double val[kCacheLines][2];
+    double val[2][kCacheLines];  // one array per feature: random lines then spread over all LDS bank pairs
     // when the workgroup streams, val and this tail together are its waves' staging slices
     uint4 stage_tail[(kScatterBlock / 64) * kStageChunk * 64 - kCacheLines];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
@@ -173,8 +173,8 @@ struct ScatterState {
 __device__ __forceinline__ void scatter_begin(ScatterState& c) {
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         c.tag[e] = -1;
-        c.val[e][0] = 0.0;
-        c.val[e][1] = 0.0;
+        c.val[0][e] = 0.0;
+        c.val[1][e] = 0.0;
     }
     for (int b = threadIdx.x; b < kMaxBins; b += kScatterBlock) c.bin_count[b] = 0u;
     if (threadIdx.x == 0) c.hits = 0u;
@@ -387,8 +387,8 @@ __device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, float* __restr
             if (miss) {
                 const int e = cache_find(c, slot[r], found);
                 if (e >= 0) {
-                    __hip_atomic_fetch_add(&c.val[e][0], static_cast<double>(x0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(&c.val[e][1], static_cast<double>(x1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&c.val[0][e], static_cast<double>(x0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&c.val[1][e], static_cast<double>(x1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     miss = false;
                 }
             }
@@ -414,7 +414,7 @@ __device__ __forceinline__ void cache_flush(ScatterState& c, float* __restrict__
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         const int owner = c.tag[e];
         if (owner != -1) {
-            const float v0 = static_cast<float>(c.val[e][0]), v1 = static_cast<float>(c.val[e][1]);
+            const float v0 = static_cast<float>(c.val[0][e]), v1 = static_cast<float>(c.val[1][e]);
             const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
             if (!binned) {
                 float* g = level_grad + 2 * static_cast<size_t>(owner);
