@@ -51,6 +51,7 @@ extern "C" {
 #define PENC_ERR_MISALIGNED 5          /* lattice_values / lattice_values_grad not 8-byte aligned */
 #define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
 #define PENC_ERR_SCRATCH_TOO_SMALL 7    /* penc_backward_static: the problem does not fit the static scratch */
+#define PENC_ERR_WORKSPACE_TOO_SMALL 8  /* penc_backward_rowmajor with positions_grad: no room for the level-major copy */
 
 const char* penc_status_string(int status);
 
@@ -121,11 +122,27 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                          const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                          void* stream);
 
-/* The table gradient of penc_backward, reading the upstream gradient as the layer after the encoding
- * produces it: rows grad_rows[n][2*level + feature] of grad_row_stride floats (even, >= 2*nr_levels;
- * 8-byte aligned), instead of [level][feature][n].  lattice_values_grad is cleared first.
+/* penc_backward reading the upstream gradient as the layer after the encoding produces it: rows
+ * grad_rows[n][2*level + feature] of grad_row_stride floats (even, >= 2*nr_levels; 8-byte aligned)
+ * instead of [level][feature][n].  Same outputs and rules as penc_backward.
+ *   - The table gradient reads the rows in place.
+ *   - The position gradient gathers level by level and needs its upstream gradient in
+ *     [level][feature][n] order: that copy (8*nr_levels*nr_positions bytes) is kept at the front of the
+ *     workspace.  When the table gradient is wanted too, the scattering kernel writes it as a
+ *     by-product of reading the rows; otherwise the rows are transposed first.  With positions_grad the
+ *     workspace is therefore required: penc_backward_rowmajor_workspace_bytes() gives the size that also
+ *     serves the scatter and the partial sums; PENC_ERR_WORKSPACE_TOO_SMALL if the copy does not fit.
  * Replaces: the strided `.contiguous()` copy of src/pytorch_modules/funcs.py:47 followed by
- * Encoding<D,2>::backward with only require_lattice_values_grad set (src/Encoding.cu:112-215). */
+ * Encoding<D,2>::backward (src/Encoding.cu:112-215). */
+size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
+                                              int want_lattice_values_grad, int want_positions_grad);
+int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                           const float* positions, const float* lattice_values, const float* scale_factor,
+                           const float* random_shift, const float* anneal_window, const float* grad_rows,
+                           int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* penc_backward_rowmajor for the table gradient alone (lattice_values is not needed). */
 int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
                                  const float* positions, const float* scale_factor, const float* random_shift,
                                  const float* anneal_window, const float* grad_rows, int64_t grad_row_stride,
@@ -144,6 +161,19 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
                                         const float* grad_sliced_values, float* lattice_values_grad,
                                         float* grad_grad_sliced_values, int concat_points, void* workspace,
                                         size_t workspace_bytes, void* stream);
+
+/* penc_double_backward_from_positions with the upstream gradient of the first backward given as rows
+ * grad_rows[n][2*level + feature] (see penc_backward_rowmajor), read in place by the scattering half.
+ * grad_grad_sliced_values is written as [L+E][2][N] like before.
+ * Replaces: the same reference code as penc_double_backward_from_positions, fed by funcs.py:47's copy. */
+int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
+                                                 int capacity, const float* positions, const float* lattice_values,
+                                                 const float* scale_factor, const float* random_shift,
+                                                 const float* anneal_window, const float* double_positions_grad,
+                                                 const float* grad_rows, int64_t grad_row_stride,
+                                                 float* lattice_values_grad, float* grad_grad_sliced_values,
+                                                 int concat_points, void* workspace, size_t workspace_bytes,
+                                                 void* stream);
 
 /* dst[c][r] = src[r][c] for a dense row-major rows x cols matrix with cols <= 255 (2 * levels):
  * turns the row-major upstream gradient (N, 2(L+E)) into the grad_sliced_values layout

@@ -36,6 +36,16 @@ _SIGNATURES = {
     "penc_backward_static": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                             _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                             ctypes.c_void_p]),
+    "penc_backward_rowmajor_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                                 ctypes.c_int, ctypes.c_int]),
+    "penc_backward_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                              _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
+                                              _c_f32p, _c_f32p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_double_backward_from_positions_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                                                    ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                                                    _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
+                                                                    _c_f32p, ctypes.c_int, ctypes.c_void_p,
+                                                                    ctypes.c_size_t, ctypes.c_void_p]),
     "penc_backward_table_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                                     _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
                                                     ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
@@ -90,24 +100,54 @@ def scale_factors(pos_dim, sigmas):
     return out
 
 
-# Levels binned per pass by the table-gradient scatter (0: the library's default, < 0: no workspace,
-# i.e. direct atomics).  The workspace is taken from torch's caching allocator for the duration of a call.
+# Levels binned per pass by the table-gradient scatter (0: the library's default, all levels in one pass;
+# < 0: no workspace, i.e. direct atomics).  The workspace is taken from torch's caching allocator for
+# the duration of a call.  Its size grows with points x levels (about 1.4 GiB for 2^20 points, 24
+# levels, pos_dim 3): MAX_WORKSPACE_BYTES caps the request, and a request the allocator cannot serve
+# is retried with fewer levels per pass and finally without a workspace; the library computes the
+# same sums either way (more passes over the levels, or direct atomics).
 LEVELS_PER_PASS = 0
+MAX_WORKSPACE_BYTES = None
 
 
-def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device, table_grad=True, positions_grad=False):
-    """Scratch memory for one gradient call (None when the library would not use any)."""
-    if LEVELS_PER_PASS < 0:
+def _scatter_bytes(pos_dim, nr_positions, nr_levels, capacity, levels_per_pass):
+    return int(lib().penc_scatter_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels), int(capacity),
+                                                  int(levels_per_pass)))
+
+
+def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device, table_grad=True, positions_grad=False,
+                      fixed_bytes=0, required_bytes=0):
+    """Scratch memory for one gradient call (None when the library would not use any).
+
+    ``fixed_bytes`` is added to every request (the level-major copy of a row-major upstream gradient);
+    ``required_bytes`` is the part of it the call cannot do without."""
+    if LEVELS_PER_PASS < 0 and not required_bytes:
         return None
-    nbytes = 0
-    if table_grad:
-        nbytes = int(lib().penc_scatter_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels), int(capacity),
-                                                        int(LEVELS_PER_PASS)))
+    pos_bytes = 0
     if positions_grad:
-        nbytes = max(nbytes, int(lib().penc_positions_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels))))
-    if nbytes == 0:
-        return None
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+        pos_bytes = int(lib().penc_positions_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels)))
+    per_pass = nr_levels if LEVELS_PER_PASS <= 0 else min(LEVELS_PER_PASS, nr_levels)
+    if not table_grad or LEVELS_PER_PASS < 0:
+        per_pass = 0
+    while True:
+        nbytes = _scatter_bytes(pos_dim, nr_positions, nr_levels, capacity, per_pass) if per_pass else 0
+        nbytes = max(nbytes, pos_bytes) + fixed_bytes
+        over_cap = MAX_WORKSPACE_BYTES is not None and nbytes > MAX_WORKSPACE_BYTES
+        if not over_cap:
+            if nbytes == 0:
+                return None
+            try:
+                return torch.empty(nbytes, dtype=torch.uint8, device=device)
+            except torch.cuda.OutOfMemoryError:
+                pass
+        if per_pass > 1:
+            per_pass //= 2      # fewer levels per pass: a smaller workspace, more passes
+        elif per_pass == 1 or pos_bytes:
+            per_pass, pos_bytes = 0, 0   # no binning and no partial sums: direct atomics, one thread per point
+        elif required_bytes and fixed_bytes:
+            return torch.empty(required_bytes, dtype=torch.uint8, device=device)   # raises if even that fails
+        else:
+            return None
 
 
 def _ptr(t):
@@ -258,49 +298,63 @@ class EncodingWrapper:
 
     def backward(self, inp, grad_sliced_values_monolithic):
         """-> (lattice_values_grad (L,C,2) or None, positions_grad (N,D) or None)
-        (reference: Encoding<D,2>::backward, src/Encoding.cu:112-215)."""
+        (reference: Encoding<D,2>::backward, src/Encoding.cu:112-215).
+
+        The upstream gradient may be the contiguous (L+E, 2, N) tensor the reference asks for, or a
+        (L+E, 2, N) view of row-major rows (what autograd hands over for the module's (N, 2(L+E))
+        output, see ``is_row_major_view``): that is read as it is, with no layout copy by the caller."""
         fp = self.fixed_params
         pos, lv, shift, win, levels, cap = self._check_common(inp)
         n = pos.shape[0]
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
-        table_only = inp.m_require_lattice_values_grad and not inp.m_require_positions_grad
-        self._check_grad(grad_sliced_values_monolithic, levels, extra, n, allow_rows=table_only)
+        grad = grad_sliced_values_monolithic
+        self._check_grad(grad, levels, extra, n, allow_rows=True)
         lv_grad = torch.empty_like(lv) if inp.m_require_lattice_values_grad else None
         pos_grad = torch.empty_like(pos) if inp.m_require_positions_grad else None
         if lv_grad is None and pos_grad is None:
             return None, None
         with torch.cuda.device(pos.device):
+            if not grad.is_contiguous():  # rows (N, 2(L+E))
+                copy_bytes = 8 * levels * n + 512 if pos_grad is not None else 0
+                ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None,
+                                       fixed_bytes=copy_bytes, required_bytes=copy_bytes)
+                _check(lib().penc_backward_rowmajor(
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    _ptr(win), _ptr(grad), grad.stride(2), _ptr(lv_grad), _ptr(pos_grad), _ptr(ws),
+                    0 if ws is None else ws.numel(), _stream()), "backward")
+                return lv_grad, pos_grad
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None)
-            if not grad_sliced_values_monolithic.is_contiguous():  # rows (N, 2(L+E)): read in place, no copy
-                _check(lib().penc_backward_table_rowmajor(
-                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
-                    _ptr(grad_sliced_values_monolithic), grad_sliced_values_monolithic.stride(2), _ptr(lv_grad),
-                    _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
-                return lv_grad, None
             _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
-                                       _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
-                                       _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(pos_grad),
-                                       _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
+                                       _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(grad), _ptr(lv_grad),
+                                       _ptr(pos_grad), _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
         return lv_grad, pos_grad
 
     def double_backward_from_positions(self, inp, double_positions_grad, grad_sliced_values_monolithic):
         """-> (lattice_values_grad (L,C,2), grad_grad_sliced_values (L+E,2,N))
-        (reference: Encoding<D,2>::double_backward_from_positions, src/Encoding.cu:219-334)."""
+        (reference: Encoding<D,2>::double_backward_from_positions, src/Encoding.cu:219-334).
+        The upstream gradient of the first backward may again be a view of row-major rows."""
         fp = self.fixed_params
         pos, lv, shift, win, levels, cap = self._check_common(inp)
         n = pos.shape[0]
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
-        self._check_grad(grad_sliced_values_monolithic, levels, extra, n)
+        grad = grad_sliced_values_monolithic
+        self._check_grad(grad, levels, extra, n, allow_rows=True)
         _check_f32_gpu(double_positions_grad, "double_positions_grad", 2)
         _require(double_positions_grad.shape == pos.shape, "double_positions_grad should be nr_positions x pos_dim")
         dpos = double_positions_grad.contiguous()
         lv_grad = torch.empty_like(lv)
-        ggs = torch.empty_like(grad_sliced_values_monolithic)
+        ggs = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
         with torch.cuda.device(pos.device):
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device)
+            if not grad.is_contiguous():
+                _check(lib().penc_double_backward_from_positions_rowmajor(
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    _ptr(win), _ptr(dpos), _ptr(grad), grad.stride(2), _ptr(lv_grad), _ptr(ggs), int(fp.m_concat_points),
+                    _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "double_backward_from_positions")
+                return lv_grad, ggs
             _check(lib().penc_double_backward_from_positions(
                 self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
-                _ptr(win), _ptr(dpos), _ptr(grad_sliced_values_monolithic), _ptr(lv_grad), _ptr(ggs),
+                _ptr(win), _ptr(dpos), _ptr(grad), _ptr(lv_grad), _ptr(ggs),
                 int(fp.m_concat_points), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
                 "double_backward_from_positions")
         return lv_grad, ggs

@@ -126,6 +126,9 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 // floats (what the layer after the encoding produces) instead of [level][feature][n].  A die walks
 // all levels of a group of points back to back, so the rows mostly come from L2 (measured: fetched
 // from memory 2.7 times, not once per level) although every level only uses 8 bytes of each.
+// With `grad_level_major` the kernel also leaves the values it read in [level][feature][n] order
+// (for the position-gradient kernel, which gathers level by level and wants its upstream gradient
+// coalesced): the layout change rides on reads this kernel makes anyway.
 // kSecondOrder: the table-gradient half of the double backward (EncodingGPU.cuh:1016-1257): the
 // vertex weights are the derivatives of the barycentric weights along `double_pos_grad` instead of
 // the barycentric weights themselves; everything else is the same scatter.
@@ -136,7 +139,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
                       const float* __restrict__ grad_sliced, int64_t grad_row_stride,
-                      const float* __restrict__ double_pos_grad, float* __restrict__ table_grad, BinTarget pass_bins) {
+                      const float* __restrict__ double_pos_grad, float* __restrict__ table_grad,
+                      float* __restrict__ grad_level_major, BinTarget pass_bins) {
     __shared__ ScatterState state;
     // Workgroups are dealt round-robin to the kXcds dies, each with an L2 of its own.  The j-th
     // workgroup of a die takes level j % levels of one group of points: a die works through all
@@ -202,6 +206,13 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
         if constexpr (kSecondOrder) q_next = load_group_point(group_q, nn_next);
         float g0_next, g1_next;
         load_grad(nn_next, g0_next, g1_next);
+        if constexpr (kRowMajor) {
+            if (grad_level_major != nullptr && active) {
+                float* out = grad_level_major + (static_cast<size_t>(level) * 2) * n_points + tile_base + threadIdx.x;
+                out[0] = g0;
+                out[n_points] = g1;
+            }
+        }
         if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
@@ -371,17 +382,17 @@ simplex_debug_kernel(int n_points, uint32_t capacity, uint32_t cap_mask, const f
 constexpr int kTransposeRows = 64;  // rows per workgroup: one wavefront-wide run per written column
 
 __global__ void __launch_bounds__(kBlock)
-transpose_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t rows, int cols) {
+transpose_kernel(const float* __restrict__ src, int64_t src_row_stride, float* __restrict__ dst, int64_t rows, int cols) {
     extern __shared__ float tile[];  // kTransposeRows x (cols | 1)
     const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTransposeRows;
     const int n_rows = rows - row0 < kTransposeRows ? static_cast<int>(rows - row0) : kTransposeRows;
     const int stride = cols | 1;  // odd: a column read walks all banks
-    const float* chunk = src + row0 * cols;
+    const float* chunk = src + row0 * src_row_stride;
     const int n_values = n_rows * cols;
     int r = threadIdx.x / cols, c = threadIdx.x % cols;
     const int dr = kBlock / cols, dc = kBlock % cols;
     for (int i = threadIdx.x; i < n_values; i += kBlock) {
-        tile[r * stride + c] = chunk[i];
+        tile[r * stride + c] = chunk[r * src_row_stride + c];
         r += dr;
         c += dc;
         if (c >= cols) {
@@ -582,11 +593,13 @@ using namespace penc;
 // The table gradient of penc_backward / penc_backward_table_rowmajor: clear, scatter, reduce the
 // bins, in as many passes over the levels as the workspace asks for.  grad_row_stride == 0 means
 // the [level][feature][n] layout, otherwise the gradient is rows of that many floats.  With
-// double_pos_grad the same for the table-gradient half of the double backward (level-major only).
+// double_pos_grad the same for the table-gradient half of the double backward.  grad_level_major (rows
+// only, may be NULL) receives the upstream gradient in [level][feature][n] order as a by-product.
 static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
                           const float* scale_factor, const float* random_shift, const float* anneal_window,
                           const float* grad, int64_t grad_row_stride, const float* double_pos_grad,
-                          float* lattice_values_grad, void* workspace, size_t workspace_bytes, hipStream_t st) {
+                          float* lattice_values_grad, float* grad_level_major, void* workspace, size_t workspace_bytes,
+                          hipStream_t st) {
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
@@ -602,8 +615,10 @@ static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int 
                                                 dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
                                                 tiles_per_group, cap, mask, positions, scale_factor, random_shift,           \
                                                 anneal_window, grad, grad_row_stride, double_pos_grad, lattice_values_grad,  \
-                                                plan.target))
-        if (double_pos_grad != nullptr) {
+                                                grad_level_major, plan.target))
+        if (double_pos_grad != nullptr && grad_row_stride != 0) {
+            PENC_LAUNCH_TABLE(true, true);
+        } else if (double_pos_grad != nullptr) {
             PENC_LAUNCH_TABLE(false, true);
         } else if (grad_row_stride != 0) {
             PENC_LAUNCH_TABLE(true, false);
@@ -616,6 +631,48 @@ static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int 
             if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, lattice_values_grad, st)) return rc;
     }
     return PENC_OK;
+}
+
+// The position gradient of penc_backward / penc_backward_rowmajor from a level-major upstream gradient:
+// levels in groups of pos_levels_per_group() when the workspace can hold the partial sums, else one
+// thread per point walks all levels.
+static int positions_backward(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
+                              const float* lattice_values, const float* scale_factor, const float* random_shift,
+                              const float* anneal_window, const float* grad_level_major, float* positions_grad,
+                              void* workspace, size_t workspace_bytes, hipStream_t st) {
+    const int n = static_cast<int>(nr_positions);
+    const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
+    const size_t n_values = static_cast<size_t>(nr_positions) * pos_dim;
+    int per_group = nr_levels, groups = 1;
+    float* partial = positions_grad;
+    const uintptr_t ws = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
+    const int want_groups = (nr_levels + pos_levels_per_group(pos_dim) - 1) / pos_levels_per_group(pos_dim);
+    if (workspace != nullptr && want_groups > 1 &&
+        workspace_bytes >= (ws - reinterpret_cast<uintptr_t>(workspace)) + want_groups * n_values * sizeof(float)) {
+        per_group = pos_levels_per_group(pos_dim);
+        groups = want_groups;
+        partial = reinterpret_cast<float*>(ws);
+    }
+    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions), groups),
+                                                dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
+                                                lattice_values, scale_factor, random_shift, anneal_window,
+                                                grad_level_major, partial));
+    if (int rc = check_launch()) return rc;
+    if (groups > 1) {
+        const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
+        hipLaunchKernelGGL(reduce_level_groups_kernel, dim3(static_cast<unsigned>(want < 8192 ? want : 8192)), dim3(kBlock),
+                           0, st, partial, groups, n_values, positions_grad);
+        if (int rc = check_launch()) return rc;
+    }
+    return PENC_OK;
+}
+
+static int transpose_rows(const float* src, int64_t src_row_stride, float* dst, int64_t rows, int cols, hipStream_t st) {
+    const size_t lds = static_cast<size_t>(kTransposeRows) * (cols | 1) * sizeof(float);
+    if (cols <= 0 || cols > 255 || lds > 64 * 1024) return PENC_ERR_BAD_SIZE;
+    const unsigned blocks = static_cast<unsigned>((rows + kTransposeRows - 1) / kTransposeRows);
+    hipLaunchKernelGGL(transpose_kernel, dim3(blocks), dim3(kBlock), lds, st, src, src_row_stride, dst, rows, cols);
+    return check_launch();
 }
 
 // penc_backward and penc_backward_static: argument checks, then the table gradient (clear, scatter,
@@ -632,38 +689,14 @@ static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
     if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
     if ((lattice_values && !aligned8(lattice_values)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int n = static_cast<int>(nr_positions);
-    const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     if (lattice_values_grad)
         if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
-                                    anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, workspace, workspace_bytes, st))
+                                    anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, nullptr, workspace,
+                                    workspace_bytes, st))
             return rc;
-    if (positions_grad) {
-        // levels in groups of pos_levels_per_group() when the workspace can hold the partial sums
-        // (the table-gradient scatter above is done with it: same stream), else one group
-        const size_t n_values = static_cast<size_t>(nr_positions) * pos_dim;
-        int per_group = nr_levels, groups = 1;
-        float* partial = positions_grad;
-        const uintptr_t ws = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
-        const int want_groups = (nr_levels + pos_levels_per_group(pos_dim) - 1) / pos_levels_per_group(pos_dim);
-        if (workspace != nullptr && want_groups > 1 &&
-            workspace_bytes >= (ws - reinterpret_cast<uintptr_t>(workspace)) + want_groups * n_values * sizeof(float)) {
-            per_group = pos_levels_per_group(pos_dim);
-            groups = want_groups;
-            partial = reinterpret_cast<float*>(ws);
-        }
-        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions), groups),
-                                                    dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
-                                                    lattice_values, scale_factor, random_shift, anneal_window,
-                                                    grad_sliced_values, partial));
-        if (int rc = check_launch()) return rc;
-        if (groups > 1) {
-            const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
-            hipLaunchKernelGGL(reduce_level_groups_kernel, dim3(static_cast<unsigned>(want < 8192 ? want : 8192)), dim3(kBlock),
-                               0, st, partial, groups, n_values, positions_grad);
-            if (int rc = check_launch()) return rc;
-        }
-    }
+    if (positions_grad)
+        return positions_backward(pos_dim, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+                                  random_shift, anneal_window, grad_sliced_values, positions_grad, workspace, workspace_bytes, st);
     return PENC_OK;
 }
 
@@ -678,6 +711,7 @@ const char* penc_status_string(int status) {
         case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2 since other values are not implemented";
         case PENC_ERR_MISALIGNED: return "lattice_values and lattice_values_grad must be 8-byte aligned";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
+        case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major copy of the upstream gradient (penc_backward_rowmajor_workspace_bytes)";
         case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
         default: return "unknown status";
     }
@@ -774,34 +808,87 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                          PENC_STATIC_SCRATCH_BYTES, stream);
 }
 
+static int check_rows(const float* grad_rows, int64_t grad_row_stride, int64_t nr_positions, int nr_levels) {
+    if (!grad_rows) return PENC_ERR_NULL_POINTER;
+    if (grad_row_stride < 2 * static_cast<int64_t>(nr_levels) || (grad_row_stride & 1) != 0 ||
+        grad_row_stride * nr_positions >= (int64_t{1} << 31))
+        return PENC_ERR_BAD_SIZE;
+    if (!aligned8(grad_rows)) return PENC_ERR_MISALIGNED;
+    return PENC_OK;
+}
+
+size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
+                                              int want_lattice_values_grad, int want_positions_grad) {
+    if (pos_dim < 2 || pos_dim > 8 || nr_positions <= 0 || nr_levels <= 0 || capacity <= 0) return 0;
+    size_t scratch = 0;
+    if (want_lattice_values_grad) scratch = penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels, capacity, 0);
+    if (!want_positions_grad) return scratch;
+    const size_t partial = penc_positions_workspace_bytes(pos_dim, nr_positions, nr_levels);
+    const size_t copy = static_cast<size_t>(nr_levels) * 2 * static_cast<size_t>(nr_positions) * sizeof(float);
+    return 512 + copy + (scratch > partial ? scratch : partial);
+}
+
+int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                           const float* positions, const float* lattice_values, const float* scale_factor,
+                           const float* random_shift, const float* anneal_window, const float* grad_rows,
+                           int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
+    if (!positions || !scale_factor || !random_shift || !anneal_window) return PENC_ERR_NULL_POINTER;
+    if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
+    if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
+    if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels)) return rc;
+    if ((lattice_values && !aligned8(lattice_values)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (!positions_grad)
+        return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+                              anneal_window, grad_rows, grad_row_stride, nullptr, lattice_values_grad, nullptr, workspace,
+                              workspace_bytes, st);
+    // The position gradient gathers level by level and reads its upstream gradient as [level][feature][n]:
+    // that copy lives at the front of the workspace; the rest serves the scatter and then the partial sums.
+    const size_t copy_bytes = static_cast<size_t>(nr_levels) * 2 * static_cast<size_t>(nr_positions) * sizeof(float);
+    const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
+    const size_t lost = base - reinterpret_cast<uintptr_t>(workspace);
+    if (workspace == nullptr || workspace_bytes < lost + copy_bytes) return PENC_ERR_WORKSPACE_TOO_SMALL;
+    float* level_major = reinterpret_cast<float*>(base);
+    const size_t copy_span = (copy_bytes + 255u) & ~size_t{255};
+    void* rest = workspace_bytes >= lost + copy_span + 256 ? reinterpret_cast<void*>(base + copy_span) : nullptr;
+    const size_t rest_bytes = rest ? workspace_bytes - lost - copy_span : 0;
+    if (lattice_values_grad) {
+        // the scattering kernel reads every (point, level) pair of the rows anyway and leaves the copy behind
+        if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+                                    anneal_window, grad_rows, grad_row_stride, nullptr, lattice_values_grad, level_major,
+                                    rest, rest_bytes, st))
+            return rc;
+    } else {
+        const int cols = 2 * nr_levels;
+        if (cols > 255) return PENC_ERR_BAD_SIZE;
+        if (int rc = transpose_rows(grad_rows, grad_row_stride, level_major, nr_positions, cols, st)) return rc;
+    }
+    return positions_backward(pos_dim, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+                              random_shift, anneal_window, level_major, positions_grad, rest, rest_bytes, st);
+}
+
 int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
                                  const float* positions, const float* scale_factor, const float* random_shift,
                                  const float* anneal_window, const float* grad_rows, int64_t grad_row_stride,
                                  float* lattice_values_grad, void* workspace, size_t workspace_bytes, void* stream) {
-    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
-    if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_rows || !lattice_values_grad)
-        return PENC_ERR_NULL_POINTER;
-    if (grad_row_stride < 2 * static_cast<int64_t>(nr_levels) || (grad_row_stride & 1) != 0 ||
-        grad_row_stride * nr_positions >= (int64_t{1} << 31))
-        return PENC_ERR_BAD_SIZE;
-    if (!aligned8(lattice_values_grad) || !aligned8(grad_rows)) return PENC_ERR_MISALIGNED;
-    return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
-                          grad_rows, grad_row_stride, nullptr, lattice_values_grad, workspace, workspace_bytes,
-                          static_cast<hipStream_t>(stream));
+    if (!lattice_values_grad) return PENC_ERR_NULL_POINTER;
+    return penc_backward_rowmajor(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, nullptr, scale_factor,
+                                  random_shift, anneal_window, grad_rows, grad_row_stride, lattice_values_grad, nullptr,
+                                  workspace, workspace_bytes, stream);
 }
 
-int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
-                                        int capacity, const float* positions,
-                                        const float* lattice_values, const float* scale_factor,
-                                        const float* random_shift, const float* anneal_window,
-                                        const float* double_positions_grad,
-                                        const float* grad_sliced_values, float* lattice_values_grad,
-                                        float* grad_grad_sliced_values, int concat_points, void* workspace,
-                                        size_t workspace_bytes, void* stream) {
+static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                const float* positions, const float* lattice_values, const float* scale_factor,
+                                const float* random_shift, const float* anneal_window,
+                                const float* double_positions_grad, const float* grad, int64_t grad_row_stride,
+                                float* lattice_values_grad, float* grad_grad_sliced_values, int concat_points,
+                                void* workspace, size_t workspace_bytes, void* stream) {
     const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
     if (!positions || !lattice_values || !scale_factor || !random_shift || !anneal_window ||
-        !double_positions_grad || !grad_sliced_values)
+        !double_positions_grad || !grad)
         return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !grad_grad_sliced_values) return PENC_ERR_NULL_POINTER;
     if (!aligned8(lattice_values) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
@@ -817,17 +904,44 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
     }
     if (!lattice_values_grad) return PENC_OK;
     return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
-                          grad_sliced_values, 0, double_positions_grad, lattice_values_grad, workspace, workspace_bytes, st);
+                          grad, grad_row_stride, double_positions_grad, lattice_values_grad, nullptr, workspace,
+                          workspace_bytes, st);
+}
+
+int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
+                                        int capacity, const float* positions,
+                                        const float* lattice_values, const float* scale_factor,
+                                        const float* random_shift, const float* anneal_window,
+                                        const float* double_positions_grad,
+                                        const float* grad_sliced_values, float* lattice_values_grad,
+                                        float* grad_grad_sliced_values, int concat_points, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values,
+                                scale_factor, random_shift, anneal_window, double_positions_grad, grad_sliced_values, 0,
+                                lattice_values_grad, grad_grad_sliced_values, concat_points, workspace, workspace_bytes,
+                                stream);
+}
+
+int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
+                                                 int capacity, const float* positions, const float* lattice_values,
+                                                 const float* scale_factor, const float* random_shift,
+                                                 const float* anneal_window, const float* double_positions_grad,
+                                                 const float* grad_rows, int64_t grad_row_stride,
+                                                 float* lattice_values_grad, float* grad_grad_sliced_values,
+                                                 int concat_points, void* workspace, size_t workspace_bytes,
+                                                 void* stream) {
+    if (nr_levels > 0 && nr_positions > 0)
+        if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels)) return rc;
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values,
+                                scale_factor, random_shift, anneal_window, double_positions_grad, grad_rows,
+                                grad_row_stride, lattice_values_grad, grad_grad_sliced_values, concat_points, workspace,
+                                workspace_bytes, stream);
 }
 
 int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream) {
     if (!src || !dst) return PENC_ERR_NULL_POINTER;
     if (rows <= 0 || cols <= 0 || cols > 255 || rows > ((int64_t{1} << 31) - 1) / cols) return PENC_ERR_BAD_SIZE;
-    const size_t lds = static_cast<size_t>(kTransposeRows) * (cols | 1) * sizeof(float);
-    if (lds > 64 * 1024) return PENC_ERR_BAD_SIZE;
-    const unsigned blocks = static_cast<unsigned>((rows + kTransposeRows - 1) / kTransposeRows);
-    hipLaunchKernelGGL(transpose_kernel, dim3(blocks), dim3(kBlock), lds, static_cast<hipStream_t>(stream), src, dst, rows, cols);
-    return check_launch();
+    return transpose_rows(src, cols, dst, rows, cols, static_cast<hipStream_t>(stream));
 }
 
 int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,

@@ -246,7 +246,8 @@ def test_row_major_entry_point_rejects_bad_strides():
 
 
 def test_module_backward_reads_the_upstream_gradient_in_place():
-    """Table-only training takes no layout copy at all; with position gradients the copy is made."""
+    """A row-major upstream gradient reaches the library as it is: neither table-only training nor the
+    path with position gradients and a double backward (the SDF path) makes a layout copy first."""
     import permutohedral_encoding_amd as pe
     from permutohedral_encoding_amd import _native
     torch.manual_seed(3)
@@ -260,11 +261,76 @@ def test_module_backward_reads_the_upstream_gradient_in_place():
     try:
         enc(pts).backward(up)
         g_table_only = enc.lattice_values.grad.clone()
-        assert calls == []
         enc.lattice_values.grad = None
         pts_g = pts.clone().requires_grad_(True)
-        enc(pts_g).backward(up)
-        assert calls == [1]
+        out = enc(pts_g)
+        grad_pos, = torch.autograd.grad(out, pts_g, up, create_graph=True)
+        g_table = enc.lattice_values.grad
+        assert g_table is None  # autograd.grad with inputs=[pts_g] leaves the parameter alone
+        (grad_pos ** 2).sum().backward()   # double backward from the row-major gradient saved by the first backward
+        assert calls == []
     finally:
         _native_funcs.level_major_gradient = real
-    assert torch.allclose(g_table_only, enc.lattice_values.grad, rtol=1e-3, atol=1e-6 * g_table_only.abs().max().item())
+    # the same through the level-major copy the reference would make
+    pts_c = pts.clone().requires_grad_(True)
+    enc2 = pe.PermutoEncoding(3, 1 << 14, 8, 2, np.geomspace(1.0, 1e-3, 8))
+    enc2.load_state_dict(enc.state_dict())
+    sliced = pe.funcs.PermutoEncodingFunc.apply(enc2.lattice, enc2.lattice_values, pts_c, enc2.anneal_window, True, True)
+    up_lm = up.reshape(5000, 8, 2).permute(1, 2, 0).contiguous()
+    grad_pos_c, = torch.autograd.grad(sliced, pts_c, up_lm, create_graph=True)
+    assert torch.equal(grad_pos.detach(), grad_pos_c.detach())  # same kernel, same level-major values
+    (grad_pos_c ** 2).sum().backward()
+    a, b = enc.lattice_values.grad, enc2.lattice_values.grad
+    assert torch.allclose(a, b, rtol=1e-3, atol=1e-6 * b.abs().max().item())
+    enc2.lattice_values.grad = None
+    enc2(pts).backward(up)
+    assert torch.allclose(g_table_only, enc2.lattice_values.grad, rtol=1e-3, atol=1e-6 * g_table_only.abs().max().item())
+
+
+@pytest.mark.parametrize("d,n,levels,cap,concat", [(3, 20000, 7, 1 << 15, False), (4, 9000, 5, 50000, True), (8, 3000, 3, 1 << 12, False)])
+def test_all_gradients_from_row_major_upstream_gradient(d, n, levels, cap, concat):
+    """penc_backward_rowmajor and penc_double_backward_from_positions_rowmajor against the oracle: table
+    gradient, position gradient (from the level-major copy the scattering kernel leaves behind, or from
+    the transposed rows when the table gradient is not wanted), second-order table gradient, grad-grad."""
+    from permutohedral_encoding_amd import _native
+    from helpers import random_problem, assert_sum_close, make_encoding, gpu_input
+    p = random_problem(d, n, levels, cap, seed=43, sigma_range=(1.0, 1e-3))
+    enc, fp = make_encoding(d, p["sigmas"], p["shift"], concat_points=concat)
+    extra = _native.extra_levels(d, 2, concat)
+    cols = 2 * (levels + extra)
+    rng = np.random.default_rng(6)
+    rows = torch.from_numpy(rng.standard_normal((n, cols + 4)).astype(np.float32)).cuda()   # padded rows
+    view = rows[:, :cols].reshape(n, levels + extra, 2).permute(1, 2, 0)
+    assert _native.is_row_major_view(view)
+    sf = orc.scale_factors(d, p["sigmas"])
+    level_major = np.ascontiguousarray(view[:levels].cpu().numpy())
+    want_t = orc.backward_table(p["pos"], sf, p["shift"], p["window"], level_major, cap, want_abs=True)
+    want_p = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], level_major)
+    for need_table in (True, False):
+        tg, pg = enc.backward(gpu_input(p, need_table, True), view)
+        if need_table:
+            assert_sum_close(tg.cpu().numpy(), want_t["grad64"], want_t["abs64"], 1e-4, "table gradient from rows")
+        else:
+            assert tg is None
+        err = np.abs(pg.cpu().numpy() - want_p["grad64"])
+        assert np.all(err <= 1e-6 * want_p["abs64"] + 1e-30), "position gradient from rows"
+    tg2, ggs = enc.double_backward_from_positions(gpu_input(p), to_gpu(p["dpos"]), view)
+    want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], level_major,
+                               concat_points=concat, want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], 1e-4, "second-order table gradient from rows")
+    assert ggs.is_contiguous() and np.array_equal(ggs.cpu().numpy(), want["ggs"])
+
+
+def test_row_major_backward_needs_room_for_the_copy():
+    from permutohedral_encoding_amd import _native
+    lib = _native.lib()
+    n, levels, cap, d = 1000, 4, 256, 3
+    t = torch.zeros(n * 8, device="cuda")
+    ws = torch.empty(4096, dtype=torch.uint8, device="cuda")
+    need = lib.penc_backward_rowmajor_workspace_bytes(d, n, levels, cap, 1, 1)
+    assert need >= 8 * levels * n
+    assert lib.penc_backward_rowmajor_workspace_bytes(d, n, levels, cap, 1, 0) == lib.penc_scatter_workspace_bytes(d, n, levels, cap, 0)
+    rc = lib.penc_backward_rowmajor(d, 2, n, levels, cap, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(),
+                                    t.data_ptr(), 8, t.data_ptr(), t.data_ptr(), ws.data_ptr(), 4096,
+                                    torch.cuda.current_stream().cuda_stream)
+    assert rc == 8 and b"level-major copy" in lib.penc_status_string(rc)
