@@ -10,9 +10,16 @@ every input already resident in HBM.  Prints ONE JSON line:
                duration, measured with events on the launch stream inside the timed loop
   cpu_baseline the CPU oracle (a scalar-code OpenMP port of the reference kernels) timed on this
                machine's host cores on a bounded sample of the same workload
-  probes       measured streaming / random-gather / random-atomic rates of this GPU, which are what
-               the table traffic is really bounded by; hbm_traffic_rate relates the measured HBM
-               bytes of each phase to them
+  probes       measured streaming / random-gather / random-atomic rates of this GPU
+  measured_roofline
+               per phase, a lower bound of the phase's time built from measurements of this GPU in
+               this run: the slots every level really touches are replayed through a gather-only
+               probe (minus the same probe with all slots equal, which keeps its streaming but takes
+               the gathers out), next to the time to stream the phase's compulsory bytes at the copy
+               probe's rate and the time to issue the kernels' vector instructions; frac = bound /
+               measured, at most 1
+  hbm_traffic_rate
+               HBM bytes per launch from hardware counters (profiles/hbm_traffic.json) / phase time
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu]
 """
@@ -29,6 +36,17 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def kernel_source_digest():
+    """Identifies the kernel sources a counter summary was taken with (a summary of other sources is stale)."""
+    import hashlib
+    h = hashlib.sha1()
+    csrc = os.path.join(ROOT, "permutohedral_encoding_amd", "csrc")
+    for name in ("penc_kernels.hip", "penc_scatter.hpp", "penc_lattice.hpp"):
+        with open(os.path.join(csrc, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
 
 
 def algorithmic_bytes(w):
@@ -73,27 +91,33 @@ def cpu_baseline(w, inputs, sample_points, reps=5):
 def module_level(torch, w, inputs, steps, warmup):
     """The same step through the PyTorch module and autograd, as a user of the package pays it: output
     allocation, the (N, 2L) view, a row-major upstream gradient of shape (N, 2L) and, if the workload
-    has them, position gradients.  Not part of `value`."""
+    has them, position gradients and the double backward of an eikonal-style loss.  Not part of `value`."""
     import permutohedral_encoding_amd as pe
     enc = pe.PermutoEncoding(w.pos_dim, w.capacity, w.nr_levels, 2, inputs["sigmas"])
     with torch.no_grad():
         enc.lattice_values.copy_(torch.from_numpy(inputs["table"]))
         enc.random_shift_per_level.copy_(torch.from_numpy(inputs["shift"]))
     pos = torch.from_numpy(inputs["pos"]).cuda()
-    if "backward_pos" in w.phases:
+    sdf_like = "double_backward" in w.phases
+    if sdf_like or "backward_pos" in w.phases:
         pos.requires_grad_(True)
     window = torch.from_numpy(inputs["window"]).cuda()
     upstream = torch.from_numpy(np.ascontiguousarray(inputs["grad"].transpose(2, 0, 1).reshape(w.nr_points, -1))).cuda()
+    q = torch.from_numpy(inputs["dpos"]).cuda()
     backward = any(p.startswith("backward") for p in w.phases)
 
     def step():
-        if backward:
+        if sdf_like:
+            out = enc(pos, window)
+            grad_pos, = torch.autograd.grad(out, pos, upstream, create_graph=True)
+            (grad_pos * q).sum().backward()
+        elif backward:
             enc(pos, window).backward(upstream)
-            enc.lattice_values.grad = None
-            pos.grad = None
         else:
             with torch.no_grad():
                 enc(pos, window)
+        enc.lattice_values.grad = None
+        pos.grad = None
 
     for _ in range(warmup):
         step()
@@ -103,32 +127,37 @@ def module_level(torch, w, inputs, steps, warmup):
         step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) / steps * 1e3
-    return {"ms_per_step": ms, "point_levels_per_s": w.point_levels / (ms * 1e-3),
-            "what": "PermutoEncoding forward" + (" + autograd backward from a row-major (N, 2L) upstream gradient" if backward else "")}
+    what = "PermutoEncoding forward"
+    if sdf_like:
+        what += " + autograd.grad w.r.t. positions (create_graph) from a row-major (N, 2L) upstream gradient + backward of <grad_pos, q>"
+    elif backward:
+        what += " + autograd backward from a row-major (N, 2L) upstream gradient"
+    return {"ms_per_step": ms, "point_levels_per_s": w.point_levels / (ms * 1e-3), "what": what}
 
 
-def run_probes(torch, native, capacity, n_threads, per_thread):
+def _timed(torch, fn, iters=20, warm=3):
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters * 1e-3
+
+
+def run_probes(torch, capacity, n_threads, per_thread):
     """Streaming copy, random 8-byte gathers and random fp32 atomic pairs over one level-sized slice."""
-    lib = native.lib()
+    from permutohedral_encoding_amd import probes
+    lib = probes.lib()
     st = lambda: torch.cuda.current_stream().cuda_stream
     dev = "cuda"
     res = {}
-
-    def timed(fn, iters=20):
-        for _ in range(3):
-            fn()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / iters * 1e-3
-
     n4 = 1 << 26  # 1 GiB each way
     src = torch.empty(n4 * 4, dtype=torch.float32, device=dev).normal_()
     dst = torch.empty_like(src)
-    t = timed(lambda: lib.penc_probe_copy(src.data_ptr(), dst.data_ptr(), n4, st()))
+    t = _timed(torch, lambda: lib.penc_probe_copy(src.data_ptr(), dst.data_ptr(), n4, st()))
     res["copy_GBps"] = 2 * n4 * 16 / t / 1e9
     del src, dst
 
@@ -137,12 +166,73 @@ def run_probes(torch, native, capacity, n_threads, per_thread):
     idx = torch.randint(0, capacity, (per_thread, n_threads), dtype=torch.int32, device=dev, generator=g)
     table = torch.zeros(capacity * 2, dtype=torch.float32, device=dev)
     out = torch.empty(n_threads * 2, dtype=torch.float32, device=dev)
-    t = timed(lambda: lib.penc_probe_gather(table.data_ptr(), idx.data_ptr(), n_threads, per_thread, out.data_ptr(), st()))
+    t = _timed(torch, lambda: lib.penc_probe_gather(table.data_ptr(), idx.data_ptr(), n_threads, per_thread, out.data_ptr(), st()))
     res["gather_Gacc_per_s"] = n_threads * per_thread / t / 1e9
-    t = timed(lambda: lib.penc_probe_scatter(table.data_ptr(), idx.data_ptr(), n_threads, per_thread, st()))
+    t = _timed(torch, lambda: lib.penc_probe_scatter(table.data_ptr(), idx.data_ptr(), n_threads, per_thread, st()))
     res["scatter_Gatomic_per_s"] = 2 * n_threads * per_thread / t / 1e9
     res["slice_bytes"] = capacity * 8
     return res
+
+
+def gather_pattern_seconds(torch, native, w, fp, table, pos):
+    """Per level: what the D+1 gathers per point cost on this memory system for the slots the workload
+    really touches.  The slots (penc_simplex_debug, the forward's own device routine) are replayed
+    through the gather-only probe; the same probe with every slot equal to 0 has the same streaming
+    traffic (index reads, one store per point) but cache-resident gathers, and is subtracted."""
+    from permutohedral_encoding_amd import probes
+    lib, plib = native.lib(), probes.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    n, d, levels, cap = w.nr_points, w.pos_dim, w.nr_levels, w.capacity
+    out = torch.empty(n * 2, dtype=torch.float32, device="cuda")
+    zeros = torch.zeros((d + 1, n), dtype=torch.int32, device="cuda")
+    level_table = table[0]
+    t_zero = _timed(torch, lambda: plib.penc_probe_gather(level_table.data_ptr(), zeros.data_ptr(), n, d + 1, out.data_ptr(), st), iters=10)
+    slot = torch.empty((1, n, d + 1), dtype=torch.int32, device="cuda")
+    result = []
+    for l in range(levels):
+        rc = lib.penc_simplex_debug(d, n, 1, cap, pos.data_ptr(), fp.m_scale_factor[l:l + 1].contiguous().data_ptr(),
+                                    fp.m_random_shift_per_level[l:l + 1].contiguous().data_ptr(), 1, None, None,
+                                    slot.data_ptr(), None, st)
+        assert rc == 0, rc
+        idx = slot[0].t().contiguous()
+        level_table = table[l]
+        t_real = _timed(torch, lambda: plib.penc_probe_gather(level_table.data_ptr(), idx.data_ptr(), n, d + 1, out.data_ptr(), st), iters=10)
+        result.append(max(t_real - t_zero, 0.0))
+    return result, t_zero
+
+
+VALU_WAVE_INSTR_PER_S = 256 * 4 * 2.4e9 / 4  # 256 CUs x 4 SIMDs, one wave64 vector instruction per 4 clocks at 2.4 GHz
+
+
+def measured_roofline(w, phases, window, gather_s, copy_GBps, valu_per_point_level):
+    """Lower bound per phase = sum over levels of max(gather pattern, compulsory streaming, vector issue).
+    Every term is a lower bound of what the level costs, so the sum is one for the phase."""
+    d, l, c, n = w.pos_dim, w.nr_levels, w.capacity, w.nr_points
+    copy = copy_GBps * 1e9
+    pos_bytes = 4.0 * d * n / l
+    out = {}
+    for name, _ in phases:
+        # (slot-access passes over the table, streamed bytes per level) of the phase
+        if name == "forward":
+            passes, stream = 1, 8.0 * n + pos_bytes
+        elif name == "backward":
+            has_table, has_pos = "backward_table" in w.phases, "backward_pos" in w.phases
+            passes = int(has_table) + int(has_pos)
+            stream = (8.0 * n + pos_bytes) * passes + (8.0 * c if has_table else 0.0) + (4.0 * d * n / l if has_pos else 0.0)
+        else:
+            passes, stream = 2, 2 * (8.0 * n + 2 * pos_bytes) + 8.0 * n + 8.0 * c
+        valu = valu_per_point_level.get(name)
+        total = 0.0
+        for level in range(l):
+            if window[level] == 0.0:
+                total += (8.0 * n / copy) if name == "forward" else 0.0   # masked levels still store their zeros
+                continue
+            terms = [passes * gather_s[level], stream / copy]
+            if valu:
+                terms.append(valu * n / 64.0 / VALU_WAVE_INSTR_PER_S)
+            total += max(terms)
+        out[name] = total * 1e3
+    return out
 
 
 def main():
@@ -254,13 +344,30 @@ def main():
                     "double_backward": "grad_grad_kernel+fill_zero_kernel+backward_table_kernel<second order>+bin_reduce_kernel"}
     dominant = max(phase_ms, key=phase_ms.get)
     achieved = phase_bytes[dominant] * w.point_levels / (phase_ms[dominant] * 1e-3) / 1e9
-    traffic = None
+    # HBM bytes per launch and vector instructions per point-level come from the committed counter
+    # summaries (profiles/hbm_traffic.json, written from rocprofv3 --pmc runs of this script); an entry
+    # taken with other kernels than the ones this phase launches now is stale and is not used.
+    per_phase, valu_per_point_level = {}, {}
     traffic_file = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    traffic_note = "no counter summary for this workload under profiles/"
     if os.path.exists(traffic_file):
         with open(traffic_file) as f:
-            traffic = json.load(f).get(w.name, {}).get(dominant)
+            recorded = json.load(f)
+        if recorded.get("source_digest") != kernel_source_digest():
+            traffic_note = "profiles/hbm_traffic.json was taken with other kernel sources (stale): not used"
+            recorded = {}
+        elif w.name in recorded:
+            traffic_note = f"profiles/hbm_traffic.json, commit {recorded.get('commit', '?')}"
+        recorded = recorded.get(w.name, {})
+        for name in phase_ms:
+            entry = recorded.get(name)
+            if entry and entry.get("kernels") == kernel_names[name]:
+                per_phase[name] = entry["hbm_bytes"]
+                if entry.get("valu_wave_instr"):
+                    valu_per_point_level[name] = entry["valu_wave_instr"] * 64.0 / w.point_levels
     roofline = {"bound": "hbm", "kernel": kernel_names[dominant], "achieved": achieved, "peak": HBM_PEAK_GBPS,
-                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+                "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": per_phase.get(dominant),
+                "traffic_source": traffic_note,
                 "algorithmic_bytes_per_launch": phase_bytes[dominant] * w.point_levels,
                 "avg_launch_ms": phase_ms[dominant]}
 
@@ -287,31 +394,26 @@ def main():
         "roofline": roofline,
     }
     if not args.no_probes:
-        result["probes"] = run_probes(torch, _native, cap, n, d + 1)
+        result["probes"] = run_probes(torch, cap, n, d + 1)
         pr = result["probes"]
-        # The measured L2/MALL gather roofline: what the step would take if every one of the
-        # N*L*(D+1) slot accesses of each table-touching phase (gather or scatter alike) ran at the
-        # measured random 8-byte gather rate, plus the streaming traffic at the measured copy rate.
-        # frac can exceed 1: the coarse levels hit caches better than the probe's uniform indices, and
-        # the binned table backward replaces random slot accesses by streamed records.
-        table_phases = sum(1 for name, _ in phases if name == "forward" or (name == "backward" and (want_table or want_pos))
-                           or name == "double_backward") + (1 if ("backward", backward) in phases and want_table and want_pos else 0)
-        bound_s = table_phases * w.point_levels * (d + 1) / (pr["gather_Gacc_per_s"] * 1e9)
-        stream_bytes = sum(phase_bytes[name] - 8 * (d + 1) * (2 if name == "double_backward" else 1) for name, _ in phases) * w.point_levels
-        bound_s += max(stream_bytes, 0.0) / (pr["copy_GBps"] * 1e9)
-        result["measured_roofline"] = {"bound_ms": bound_s * 1e3, "frac": bound_s * 1e3 / ms_per_step,
-                                       "note": "every table slot access at the probe's random-gather rate + streaming at "
-                                               "the probe's copy rate; frac = bound / measured step"}
-        # How fast the HBM traffic each phase really makes (hardware byte counters, scaled by the copy
-        # probe, from profiles/) is moved, next to the rate the copy probe reaches for pure streaming.
-        if os.path.exists(traffic_file):
-            with open(traffic_file) as f:
-                per_phase = json.load(f).get(w.name, {})
+        gather_s, t_zero = gather_pattern_seconds(torch, _native, w, fp, inp.m_lattice_values, inp.m_positions_raw)
+        bound_ms = measured_roofline(w, phases, inputs["window"], gather_s, pr["copy_GBps"], valu_per_point_level)
+        result["measured_roofline"] = {
+            "bound_ms": bound_ms,
+            "frac": {k: bound_ms[k] / phase_ms[k] for k in bound_ms},
+            "step_bound_ms": sum(bound_ms.values()),
+            "step_frac": sum(bound_ms.values()) / sum(phase_ms.values()),
+            "gather_pattern_us_per_level": [round(x * 1e6, 2) for x in gather_s],
+            "note": "per level max(replay of the level's own slots through the gather-only probe minus the same "
+                    "probe with all slots equal, compulsory bytes at the copy probe's rate, vector instructions at "
+                    "one per 4 clocks per SIMD), summed over the levels; a table gradient or second table pass "
+                    "counts its slot accesses like gathers; frac = bound / measured phase time",
+        }
+        if per_phase:
             result["hbm_traffic_rate"] = {
                 "GBps": {k: per_phase[k] / (phase_ms[k] * 1e-3) / 1e9 for k in phase_ms if k in per_phase},
-                "copy_probe_GBps": result["probes"]["copy_GBps"],
-                "note": "measured HBM bytes per launch / measured phase time; the forward is bound by random 8-byte "
-                        "gathers (see probes.gather_Gacc_per_s), the table backward by streaming its slot-range records",
+                "copy_probe_GBps": pr["copy_GBps"],
+                "note": "HBM bytes per launch from hardware counters (profiles/) / measured phase time",
             }
     if not args.no_module:
         result["module_level"] = module_level(torch, w, inputs, args.steps, args.warmup)

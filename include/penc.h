@@ -194,18 +194,6 @@ int penc_simplex_debug(int pos_dim, int64_t nr_positions, int nr_levels, int cap
                        const float* positions, const float* scale_factor, const float* random_shift,
                        int gather_path, int* rem0, int* rank, int* slot, float* barycentric, void* stream);
 
-/* Memory-system probes used by the benchmark to measure the rooflines the encoding is priced
- * against; they have no counterpart in the reference.
- *   copy   : dst[i] = src[i] for n_float4 16-byte elements (streaming bandwidth, and the known-size
- *            kernel that hardware byte counters are scaled by)
- *   gather : every thread sums `per_thread` independent 8-byte loads table[idx[...]] and writes one
- *            8-byte result; idx holds n_threads*per_thread precomputed slots
- *   scatter: every thread issues `per_thread` pairs of fp32 atomic adds at table[idx[...]] */
-int penc_probe_copy(const float* src, float* dst, int64_t n_float4, void* stream);
-int penc_probe_gather(const float* table, const int* idx, int64_t n_threads, int per_thread,
-                      float* out, void* stream);
-int penc_probe_scatter(float* table, const int* idx, int64_t n_threads, int per_thread, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -4,7 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../../include/penc.h"
+#include "../../include/penc.h"  // status codes
+#include "../../include/penc_probes.h"
 
 namespace {
 

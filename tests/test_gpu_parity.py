@@ -446,6 +446,24 @@ def test_table_gradient_does_not_depend_on_the_workspace(ws_bytes):
     assert_sum_close(got, want["grad64"], want["abs64"], SUM_RTOL, f"double-backward table gradient, workspace {ws_bytes}")
 
 
+def test_capped_workspace_takes_more_passes_and_gives_the_same_sums():
+    from permutohedral_encoding_amd import _native
+    d, cap, n, levels = 3, 1 << 16, 1 << 17, 10
+    p = random_problem(d, n, levels, cap, seed=17, sigma_range=(1.0, 1e-3))
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    full = _native.lib().penc_scatter_workspace_bytes(d, n, levels, cap, 0)
+    for limit in (None, full // 3, 1 << 16):   # one pass, several passes, too small to bin anything
+        _native.MAX_WORKSPACE_BYTES = limit
+        try:
+            tg, pg = enc.backward(gpu_input(p), to_gpu(p["grad"]))
+        finally:
+            _native.MAX_WORKSPACE_BYTES = None
+        assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, workspace cap {limit}")
+        check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"]))
+
+
 def test_misaligned_workspace_and_odd_capacity():
     d, cap = 4, 50000  # not a multiple of the bin size: the last bin is partial
     p = random_problem(d, 20000, 6, cap, seed=8, sigma_range=(1.0, 1e-3))

@@ -16,8 +16,8 @@ from oracle import api as orc
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "penc.h")).read()
+def declared_functions(header="penc.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return re.findall(r"\b(penc_\w+)\s*\(", text)
 
@@ -29,6 +29,13 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(handle, n), f"{n} is declared in include/penc.h but not exported"
     assert set(names) == set(_native.EXPORTED_SYMBOLS)
+    assert not [n for n in names if "probe" in n]  # measurement aids live in their own library
+    from permutohedral_encoding_amd import probes
+    probe_names = declared_functions("penc_probes.h")
+    handle = ctypes.CDLL(probes.LIB_PATH)
+    for n in probe_names:
+        assert hasattr(handle, n), f"{n} is declared in include/penc_probes.h but not exported"
+    assert set(probe_names) == set(probes.EXPORTED_SYMBOLS) and len(probe_names) == 3
 
 
 def test_status_strings_and_extra_levels():
@@ -156,3 +163,44 @@ def test_workloads_are_seeded_and_shaped():
     r = np.linalg.norm(s - 0.5, axis=1)
     assert abs(r.mean() - 0.5) < 5e-3 and 0.015 < r.std() < 0.025
     assert workloads.WORKLOADS["c2"].point_levels == 25165824
+
+
+def test_workspace_request_is_capped_and_shrinks_when_memory_runs_out(monkeypatch):
+    """The scatter workspace grows with points x levels; the binding caps it and, when the allocator
+    refuses, asks again for fewer levels per pass, then for none (the library then adds directly)."""
+    import torch
+    d, n, levels, cap = 3, 1 << 20, 24, 1 << 18
+    lib = _native.lib()
+    full = lib.penc_scatter_workspace_bytes(d, n, levels, cap, 0)
+    one = lib.penc_scatter_workspace_bytes(d, n, levels, cap, 1)
+    assert full > 20 * one > 0
+    requests = []
+    limit = [None]
+
+    def fake_empty(nbytes, dtype=None, device=None):
+        requests.append(nbytes)
+        if limit[0] is not None and nbytes > limit[0]:
+            raise torch.cuda.OutOfMemoryError("simulated")
+        return torch.zeros(1, dtype=torch.uint8)  # stands for the buffer
+
+    monkeypatch.setattr(_native.torch, "empty", fake_empty)
+    assert _native.scatter_workspace(d, n, levels, cap, "cpu") is not None and requests == [full]
+    # capped: the largest power-of-two fraction of the levels whose records fit
+    requests.clear()
+    monkeypatch.setattr(_native, "MAX_WORKSPACE_BYTES", 400 << 20)
+    _native.scatter_workspace(d, n, levels, cap, "cpu")
+    assert len(requests) == 1 and one <= requests[0] <= 400 << 20
+    monkeypatch.setattr(_native, "MAX_WORKSPACE_BYTES", None)
+    # out of memory: 24 -> 12 -> 6 -> 3 -> 1 levels per pass, then nothing
+    requests.clear()
+    limit[0] = 2 * one
+    assert _native.scatter_workspace(d, n, levels, cap, "cpu") is not None
+    assert requests[0] == full and requests[-1] <= 2 * one and requests == sorted(requests, reverse=True)
+    requests.clear()
+    limit[0] = 0
+    assert _native.scatter_workspace(d, n, levels, cap, "cpu") is None
+    # the level-major copy of a row-major gradient is not optional: that request is repeated and may raise
+    requests.clear()
+    with pytest.raises(torch.cuda.OutOfMemoryError):
+        _native.scatter_workspace(d, n, levels, cap, "cpu", positions_grad=True, fixed_bytes=1000, required_bytes=1000)
+    assert requests[-1] == 1000
