@@ -11,15 +11,15 @@
  *  - Plain pointers and sizes only.  Unless a parameter says "host", every pointer is DEVICE
  *    memory of the GPU that is current on the calling thread; it is borrowed for the duration of
  *    the enqueued work.  The library never allocates or frees device memory and keeps no state.
- *  - All arrays are fp32, densely packed, row-major:
+ *  - All arrays are fp32, densely packed, row-major (F = nr_feat, the features per level):
  *        positions            [N][D]
- *        lattice_values       [L][C][2]      (8-byte aligned)
+ *        lattice_values       [L][C][F]      (aligned to one slot: 8 bytes for F = 2, 16 for F = 4)
  *        scale_factor         [L][D]         (from penc_scale_factors)
  *        random_shift         [L][D]
  *        anneal_window        [L]
- *        sliced_values        [L+E][2][N]    E = ceil(D/2) if concat_points else 0
- *        grad_sliced_values   [L+E][2][N]    (levels >= L are ignored)
- *        lattice_values_grad  [L][C][2]      (the reference returns this logical shape as a
+ *        sliced_values        [L+E][F][N]    E = ceil(D/F) if concat_points else 0
+ *        grad_sliced_values   [L+E][F][N]    (levels >= L are ignored)
+ *        lattice_values_grad  [L][C][F]      (8-byte aligned; the reference returns this logical shape as a
  *                                             permuted view of [L][2][C], src/Encoding.cu:141,204)
  *        positions_grad       [N][D]         (the reference returns this logical shape as a
  *                                             transposed view of [D][N], src/Encoding.cu:152,205)
@@ -30,7 +30,9 @@
  *    depend on it beyond the order of floating-point accumulation.
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is enqueued and
  *    the call returns without synchronising, like the reference's launches on the current stream.
- *  - D = pos_dim in 2..8, nr_feat must be 2 (reference: Encoding.cuh:139-156 supports 2..7 / 2).
+ *  - D = pos_dim in 2..8, nr_feat 2 or 4 (reference: Encoding.cuh:139-156 supports 2..7 and 2 only; its
+ *    instantiations for 4 and 8 features are commented out, src/Encoding.cu:362-363).  With four
+ *    features the table gradient treats the feature pairs (0,1) and (2,3) of a level like two levels.
  *  - Every function returns PENC_OK or one of the error codes below; penc_status_string() names it.
  */
 #ifndef PENC_H_
@@ -47,8 +49,8 @@ extern "C" {
 #define PENC_ERR_NULL_POINTER 1        /* a required pointer is NULL */
 #define PENC_ERR_BAD_SIZE 2            /* N, L or C is not positive, or a product overflows 2^31 elements */
 #define PENC_ERR_UNSUPPORTED_POS_DIM 3 /* pos_dim outside 2..8 (reference: Encoding.cuh:155) */
-#define PENC_ERR_UNSUPPORTED_NR_FEAT 4 /* nr_feat != 2 (reference: Encoding.cuh:142) */
-#define PENC_ERR_MISALIGNED 5          /* lattice_values / lattice_values_grad not 8-byte aligned */
+#define PENC_ERR_UNSUPPORTED_NR_FEAT 4 /* nr_feat not 2 or 4 (reference: Encoding.cuh:142 accepts 2 only) */
+#define PENC_ERR_MISALIGNED 5          /* lattice_values not aligned to a slot, or a gradient array not to 8 bytes */
 #define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
 #define PENC_ERR_SCRATCH_TOO_SMALL 7    /* penc_backward_static: the problem does not fit the static scratch */
 #define PENC_ERR_WORKSPACE_TOO_SMALL 8  /* penc_backward_rowmajor with positions_grad: no room for the level-major copy */
@@ -65,10 +67,16 @@ int penc_extra_levels(int pos_dim, int nr_feat, int concat_points);
  * Replaces: EncodingFixedParams::compute_scale_factor_tensor, Encoding.cuh:55-69. */
 int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* scale_factor_out);
 
-/* Suggested size of the `workspace` argument of the two gradient calls below for binning
- * `levels_per_pass` levels at a time (<= 0: the library's default); 0 when the capacity is too
- * large for binning.  No counterpart in the reference (its scatter is one atomicAdd per value,
- * EncodingGPU.cuh:409-410). */
+/* Suggested size of the `workspace` argument of the gradient calls below for binning
+ * `levels_per_pass` levels at a time (<= 0: the library's default, all of them); 0 when the capacity
+ * is too large for binning (above 2^22 slots).  `nr_levels` counts pairs of features: pass
+ * nr_levels * nr_feat / 2.  Per level the workspace holds, for each of the ceil(capacity / 8192)
+ * slot ranges and each group of 4096 or 8192 points, a 4-byte count and room for the group's
+ * expected share of the (pos_dim + 1) 12-byte records per point plus three standard deviations:
+ * about 13.5 * (pos_dim + 1) bytes per point and level (1.4 GiB for 2^20 points, 24 levels, pos_dim 3).
+ * Any smaller workspace works too: the levels are then binned in several passes, and with none the
+ * gradient is accumulated with direct atomics.  No counterpart in the reference (its scatter is one
+ * atomicAdd per value, EncodingGPU.cuh:409-410). */
 size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
                                     int levels_per_pass);
 
@@ -123,18 +131,18 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                          void* stream);
 
 /* penc_backward reading the upstream gradient as the layer after the encoding produces it: rows
- * grad_rows[n][2*level + feature] of grad_row_stride floats (even, >= 2*nr_levels; 8-byte aligned)
- * instead of [level][feature][n].  Same outputs and rules as penc_backward.
+ * grad_rows[n][nr_feat*level + feature] of grad_row_stride floats (even, >= nr_feat*nr_levels; 8-byte
+ * aligned) instead of [level][feature][n].  Same outputs and rules as penc_backward.
  *   - The table gradient reads the rows in place.
  *   - The position gradient gathers level by level and needs its upstream gradient in
- *     [level][feature][n] order: that copy (8*nr_levels*nr_positions bytes) is kept at the front of the
+ *     [level][feature][n] order: that copy (4*nr_feat*nr_levels*nr_positions bytes) is kept at the front of the
  *     workspace.  When the table gradient is wanted too, the scattering kernel writes it as a
  *     by-product of reading the rows; otherwise the rows are transposed first.  With positions_grad the
  *     workspace is therefore required: penc_backward_rowmajor_workspace_bytes() gives the size that also
  *     serves the scatter and the partial sums; PENC_ERR_WORKSPACE_TOO_SMALL if the copy does not fit.
  * Replaces: the strided `.contiguous()` copy of src/pytorch_modules/funcs.py:47 followed by
  * Encoding<D,2>::backward (src/Encoding.cu:112-215). */
-size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
+size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
                                               int want_lattice_values_grad, int want_positions_grad);
 int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
                            const float* positions, const float* lattice_values, const float* scale_factor,

@@ -1,9 +1,10 @@
 """ctypes binding over the CPU oracle library (test infrastructure; see ``penc_oracle.cpp``).
 
 All functions take and return NumPy arrays.  Layouts follow the reference's kernels:
-positions ``(N, D)``, table ``(L, C, 2)``, scale factors / shifts ``(L, D)``, window ``(L,)``,
-sliced values and their gradients ``(L [+extra], 2, N)``, table gradients ``(L, C, 2)``,
-position gradients ``(N, D)``.
+positions ``(N, D)``, table ``(L, C, F)``, scale factors / shifts ``(L, D)``, window ``(L,)``,
+sliced values and their gradients ``(L [+extra], F, N)``, table gradients ``(L, C, F)``,
+position gradients ``(N, D)``.  F, the number of features per level, is read off the table's or the
+gradient's shape (the reference supports F = 2 only).
 """
 import ctypes
 import os
@@ -50,8 +51,8 @@ def num_threads():
     return int(lib().penc_oracle_num_threads())
 
 
-def extra_levels(pos_dim, concat_points):
-    return (pos_dim + 1) // 2 if concat_points else 0
+def extra_levels(pos_dim, concat_points, nr_feat=2):
+    return (pos_dim + nr_feat - 1) // nr_feat if concat_points else 0
 
 
 def hash_key(key):
@@ -101,14 +102,14 @@ def simplex(pos, sf, shift, capacity, dtype=np.float32, with_keys=False):
 def forward(pos, table, sf, shift, window, concat_points=False, points_scaling=1.0, dtype=np.float32):
     pos, table, sf, shift, window = (_f(a, dtype) for a in (pos, table, sf, shift, window))
     n, d, l = _dims(pos, shift)
-    c = table.shape[1]
-    assert table.shape == (l, c, 2) and window.shape == (l,)
-    out = np.empty((l + extra_levels(d, concat_points), 2, pos.shape[0]), dtype)
+    c, f = table.shape[1], table.shape[2]
+    assert table.shape == (l, c, f) and window.shape == (l,)
+    out = np.empty((l + extra_levels(d, concat_points, f), f, pos.shape[0]), dtype)
     if dtype == np.float32:
-        rc = lib().penc_oracle_forward(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(out),
+        rc = lib().penc_oracle_forward(d, n, l, c, f, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(out),
                                        int(bool(concat_points)), ctypes.c_float(points_scaling))
     else:
-        rc = lib().penc_oracle_forward_f64(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(out),
+        rc = lib().penc_oracle_forward_f64(d, n, l, c, f, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(out),
                                            int(bool(concat_points)), ctypes.c_double(points_scaling))
     _check(rc, "forward")
     return out
@@ -118,17 +119,17 @@ def backward_table(pos, sf, shift, window, grad, capacity, dtype=np.float32, wan
     """Returns dict(grad32=(L,C,2) fp32 omp-atomic sum, grad64=fp64 sum, abs64=fp64 sum of |terms|)."""
     pos, sf, shift, window, grad = (_f(a, dtype) for a in (pos, sf, shift, window, grad))
     n, d, l = _dims(pos, shift)
-    c = int(capacity)
-    assert grad.shape[0] >= l and grad.shape[1:] == (2, pos.shape[0])
+    c, f = int(capacity), grad.shape[1]
+    assert grad.shape[0] >= l and grad.shape[1:] == (f, pos.shape[0])
     if dtype == np.float64:
-        g = np.zeros((l, c, 2), np.float64)
-        _check(lib().penc_oracle_backward_table_f64(d, n, l, c, _p(pos), _p(sf), _p(shift), _p(window), _p(grad), _p(g)),
+        g = np.zeros((l, c, f), np.float64)
+        _check(lib().penc_oracle_backward_table_f64(d, n, l, c, f, _p(pos), _p(sf), _p(shift), _p(window), _p(grad), _p(g)),
                "backward_table_f64")
         return dict(grad64=g)
-    g32 = np.zeros((l, c, 2), np.float32) if want32 else None
-    g64 = np.zeros((l, c, 2), np.float64) if want64 else None
-    a64 = np.zeros((l, c, 2), np.float64) if want_abs else None
-    _check(lib().penc_oracle_backward_table(d, n, l, c, _p(pos), _p(sf), _p(shift), _p(window), _p(grad),
+    g32 = np.zeros((l, c, f), np.float32) if want32 else None
+    g64 = np.zeros((l, c, f), np.float64) if want64 else None
+    a64 = np.zeros((l, c, f), np.float64) if want_abs else None
+    _check(lib().penc_oracle_backward_table(d, n, l, c, f, _p(pos), _p(sf), _p(shift), _p(window), _p(grad),
                                             _p(g32), _p(g64), _p(a64)), "backward_table")
     return dict(grad32=g32, grad64=g64, abs64=a64)
 
@@ -138,16 +139,16 @@ def backward_pos(pos, table, sf, shift, window, grad, dtype=np.float32):
     with every term replaced by its magnitude: the scale the rounding error of grad32 is relative to)."""
     pos, table, sf, shift, window, grad = (_f(a, dtype) for a in (pos, table, sf, shift, window, grad))
     n, d, l = _dims(pos, shift)
-    c = table.shape[1]
+    c, f = table.shape[1], table.shape[2]
     if dtype == np.float64:
         g = np.empty(pos.shape, np.float64)
-        _check(lib().penc_oracle_backward_pos_f64(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window),
+        _check(lib().penc_oracle_backward_pos_f64(d, n, l, c, f, _p(pos), _p(table), _p(sf), _p(shift), _p(window),
                                                   _p(grad), _p(g)), "backward_pos_f64")
         return dict(grad64=g)
     g32 = np.empty(pos.shape, np.float32)
     g64 = np.empty(pos.shape, np.float64)
     a64 = np.empty(pos.shape, np.float64)
-    _check(lib().penc_oracle_backward_pos(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(grad),
+    _check(lib().penc_oracle_backward_pos(d, n, l, c, f, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(grad),
                                           _p(g32), _p(g64), _p(a64)), "backward_pos")
     return dict(grad32=g32, grad64=g64, abs64=a64)
 
@@ -158,20 +159,20 @@ def double_backward(pos, table, sf, shift, window, double_pos_grad, grad, concat
     ggs_abs64 = the grad-of-grad chain with every term replaced by its magnitude)."""
     pos, table, sf, shift, window, q, grad = (_f(a, dtype) for a in (pos, table, sf, shift, window, double_pos_grad, grad))
     n, d, l = _dims(pos, shift)
-    c = table.shape[1]
+    c, f = table.shape[1], table.shape[2]
     assert q.shape == pos.shape
-    ggs = np.empty((l + extra_levels(d, concat_points), 2, pos.shape[0]), dtype)
+    ggs = np.empty((l + extra_levels(d, concat_points, f), f, pos.shape[0]), dtype)
     if dtype == np.float64:
-        g = np.zeros((l, c, 2), np.float64)
-        _check(lib().penc_oracle_double_backward_f64(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window),
+        g = np.zeros((l, c, f), np.float64)
+        _check(lib().penc_oracle_double_backward_f64(d, n, l, c, f, _p(pos), _p(table), _p(sf), _p(shift), _p(window),
                                                      _p(q), _p(grad), _p(g), _p(ggs), int(bool(concat_points))),
                "double_backward_f64")
         return dict(grad64=g, ggs=ggs)
-    g32 = np.zeros((l, c, 2), np.float32) if want32 else None
-    g64 = np.zeros((l, c, 2), np.float64) if want64 else None
-    a64 = np.zeros((l, c, 2), np.float64) if want_abs else None
+    g32 = np.zeros((l, c, f), np.float32) if want32 else None
+    g64 = np.zeros((l, c, f), np.float64) if want64 else None
+    a64 = np.zeros((l, c, f), np.float64) if want_abs else None
     ga64 = np.empty(ggs.shape, np.float64) if want_abs else None
-    _check(lib().penc_oracle_double_backward(d, n, l, c, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(q),
+    _check(lib().penc_oracle_double_backward(d, n, l, c, f, _p(pos), _p(table), _p(sf), _p(shift), _p(window), _p(q),
                                              _p(grad), _p(g32), _p(g64), _p(a64), _p(ggs), _p(ga64),
                                              int(bool(concat_points))),
            "double_backward")

@@ -177,9 +177,9 @@ inline void double_backward_bary_magnitude(const Simplex<D, R>& s, const R* q, c
     mB[0] += mB[D1];
 }
 
-inline int extra_levels(int pos_dim, int concat_points) {
-    // src/Encoding.cu:71-74 with val_dim = 2
-    return concat_points ? (pos_dim + 1) / 2 : 0;
+inline int extra_levels(int pos_dim, int nr_feat, int concat_points) {
+    // src/Encoding.cu:71-74: ceil(pos_dim / val_dim) extra levels carry the raw positions
+    return concat_points ? (pos_dim + nr_feat - 1) / nr_feat : 0;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -219,40 +219,47 @@ void simplex_dump(int64_t N, int L, int C, const R* pos, const R* sf, const R* s
 }
 
 // ------------------------------------------------------------------------------------------
+// The four kernels below take the number of features per level, F, as an argument.  The reference
+// instantiates F = 2 only (include/permutohedral_encoding/Encoding.cuh:139-143 rejects the rest, the
+// other instantiations are commented out at src/Encoding.cu:362-363), and its kernels are written
+// for val_dim = 2; F = 4 is the same algorithm with the feature loops two steps longer, and is
+// pinned by the same identities (the pinning tests run for both values).
+constexpr int kMaxFeat = 8;
+
+// ------------------------------------------------------------------------------------------
 // forward, ":99-254"
 // Pinned by: reproduction of affine functions on a collision-free table, constant table ->
 // window[l], one-hot table entry -> barycentric weight.
 
 template <int D, typename R>
-void forward(int64_t N, int L, int C, const R* pos, const R* table, const R* sf, const R* shift,
+void forward(int64_t N, int L, int C, int F, const R* pos, const R* table, const R* sf, const R* shift,
              const R* window, R* out, int concat_points, R points_scaling) {
     constexpr int D1 = D + 1;
-    const int extra = extra_levels(D, concat_points);
+    const int extra = extra_levels(D, F, concat_points);
     for (int l = 0; l < L; ++l) {
         const R w_lvl = window[l];
-        const R* tl = table + static_cast<int64_t>(l) * C * 2;
+        const R* tl = table + static_cast<int64_t>(l) * C * F;
 #pragma omp parallel for schedule(static)
         for (int64_t n = 0; n < N; ++n) {
             Simplex<D, R> s;
             locate_simplex<D, R>(pos + n * D, shift + l * D, sf + l * D, s);
             barycentric<D, R>(s);
-            R acc0 = 0, acc1 = 0;
+            R acc[kMaxFeat];
+            for (int f = 0; f < F; ++f) acc[f] = 0;
             for (int r = 0; r <= D; ++r) {
                 int key[D1];
                 vertex_key<D, R>(s, r, key);
-                const int h = lattice_slot<D>(key, C);
+                const int64_t h = static_cast<int64_t>(F) * lattice_slot<D>(key, C);
                 const R w = s.bary[r] * w_lvl;
-                acc0 = acc0 + tl[2 * static_cast<int64_t>(h)] * w;
-                acc1 = acc1 + tl[2 * static_cast<int64_t>(h) + 1] * w;
+                for (int f = 0; f < F; ++f) acc[f] = acc[f] + tl[h + f] * w;
             }
-            out[(static_cast<int64_t>(l) * 2 + 0) * N + n] = acc0;
-            out[(static_cast<int64_t>(l) * 2 + 1) * N + n] = acc1;
+            for (int f = 0; f < F; ++f) out[(static_cast<int64_t>(l) * F + f) * N + n] = acc[f];
         }
     }
     for (int e = 0; e < extra; ++e) {  // ":106-121"
-        for (int f = 0; f < 2; ++f) {
-            const int src = f + e * 2;
-            R* o = out + (static_cast<int64_t>(L + e) * 2 + f) * N;
+        for (int f = 0; f < F; ++f) {
+            const int src = f + e * F;
+            R* o = out + (static_cast<int64_t>(L + e) * F + f) * N;
 #pragma omp parallel for schedule(static)
             for (int64_t n = 0; n < N; ++n) o[n] = (src < D) ? pos[n * D + src] * points_scaling : static_cast<R>(0);
         }
@@ -260,47 +267,43 @@ void forward(int64_t N, int L, int C, const R* pos, const R* table, const R* sf,
 }
 
 // ------------------------------------------------------------------------------------------
-// backward w.r.t. the table, ":291-293, 385-414".  Output logical layout (L, C, 2) (the
+// backward w.r.t. the table, ":291-293, 385-414".  Output logical layout (L, C, F) (the
 // reference fills (L, 2, C) and returns the permuted view, src/Encoding.cu:141,204).
 // Pinned by: adjoint identity <forward(T), g> = <T, backward(g)>.
 
 template <int D, typename R, typename A>
-void backward_table(int64_t N, int L, int C, const R* pos, const R* sf, const R* shift, const R* window,
+void backward_table(int64_t N, int L, int C, int F, const R* pos, const R* sf, const R* shift, const R* window,
                     const R* grad, R* tgrad, A* tgrad_acc, A* tgrad_abs) {
     constexpr int D1 = D + 1;
     for (int l = 0; l < L; ++l) {
         const R w_lvl = window[l];
-        const int64_t base = static_cast<int64_t>(l) * C * 2;
+        const int64_t base = static_cast<int64_t>(l) * C * F;
 #pragma omp parallel for schedule(static)
         for (int64_t n = 0; n < N; ++n) {
             Simplex<D, R> s;
             locate_simplex<D, R>(pos + n * D, shift + l * D, sf + l * D, s);
             barycentric<D, R>(s);
-            const R g0 = grad[(static_cast<int64_t>(l) * 2 + 0) * N + n];
-            const R g1 = grad[(static_cast<int64_t>(l) * 2 + 1) * N + n];
+            R g[kMaxFeat];
+            for (int f = 0; f < F; ++f) g[f] = grad[(static_cast<int64_t>(l) * F + f) * N + n];
             for (int r = 0; r <= D; ++r) {
                 int key[D1];
                 vertex_key<D, R>(s, r, key);
-                const int64_t h = base + 2 * static_cast<int64_t>(lattice_slot<D>(key, C));
+                const int64_t h = base + static_cast<int64_t>(F) * lattice_slot<D>(key, C);
                 const R w = s.bary[r] * w_lvl;
-                const R t0 = g0 * w, t1 = g1 * w;
-                if (tgrad) {
+                for (int f = 0; f < F; ++f) {
+                    const R t = g[f] * w;
+                    if (tgrad) {
 #pragma omp atomic
-                    tgrad[h] += t0;
+                        tgrad[h + f] += t;
+                    }
+                    if (tgrad_acc) {
 #pragma omp atomic
-                    tgrad[h + 1] += t1;
-                }
-                if (tgrad_acc) {
+                        tgrad_acc[h + f] += static_cast<A>(t);
+                    }
+                    if (tgrad_abs) {
 #pragma omp atomic
-                    tgrad_acc[h] += static_cast<A>(t0);
-#pragma omp atomic
-                    tgrad_acc[h + 1] += static_cast<A>(t1);
-                }
-                if (tgrad_abs) {
-#pragma omp atomic
-                    tgrad_abs[h] += std::fabs(static_cast<A>(t0));
-#pragma omp atomic
-                    tgrad_abs[h + 1] += std::fabs(static_cast<A>(t1));
+                        tgrad_abs[h + f] += std::fabs(static_cast<A>(t));
+                    }
                 }
             }
         }
@@ -315,7 +318,7 @@ void backward_table(int64_t N, int L, int C, const R* pos, const R* sf, const R*
 // piecewise linear).
 
 template <int D, typename R, typename A>
-void backward_pos(int64_t N, int L, int C, const R* pos, const R* table, const R* sf, const R* shift,
+void backward_pos(int64_t N, int L, int C, int F, const R* pos, const R* table, const R* sf, const R* shift,
                   const R* window, const R* grad, R* pgrad, A* pgrad_acc, A* pgrad_abs) {
     constexpr int D1 = D + 1;
     const R inv = static_cast<R>(1) / static_cast<R>(D1);
@@ -326,22 +329,23 @@ void backward_pos(int64_t N, int L, int C, const R* pos, const R* table, const R
         for (int i = 0; i < D; ++i) { sum[i] = 0; sum_acc[i] = 0; sum_abs[i] = 0; }
         for (int l = 0; l < L; ++l) {
             const R w_lvl = window[l];
-            const R* tl = table + static_cast<int64_t>(l) * C * 2;
+            const R* tl = table + static_cast<int64_t>(l) * C * F;
             const R* sfl = sf + l * D;
             Simplex<D, R> s;
             locate_simplex<D, R>(pos + n * D, shift + l * D, sfl, s);
-            const R g0 = grad[(static_cast<int64_t>(l) * 2 + 0) * N + n];
-            const R g1 = grad[(static_cast<int64_t>(l) * 2 + 1) * N + n];
+            R g[kMaxFeat];
+            for (int f = 0; f < F; ++f) g[f] = grad[(static_cast<int64_t>(l) * F + f) * N + n];
             R dB[D + 2];
             A mB[D + 2];  // the same chain with every term replaced by its magnitude (the scale rounding errors are relative to)
             for (int k = 0; k <= D1; ++k) { dB[k] = 0; mB[k] = 0; }
             for (int r = 0; r <= D; ++r) {
                 int key[D1];
                 vertex_key<D, R>(s, r, key);
-                const int64_t h = 2 * static_cast<int64_t>(lattice_slot<D>(key, C));
-                dB[r] += tl[h] * w_lvl * g0;
-                dB[r] += tl[h + 1] * w_lvl * g1;
-                mB[r] = std::fabs(static_cast<A>(tl[h] * w_lvl * g0)) + std::fabs(static_cast<A>(tl[h + 1] * w_lvl * g1));
+                const int64_t h = static_cast<int64_t>(F) * lattice_slot<D>(key, C);
+                for (int f = 0; f < F; ++f) {
+                    dB[r] += tl[h + f] * w_lvl * g[f];
+                    mB[r] += std::fabs(static_cast<A>(tl[h + f] * w_lvl * g[f]));
+                }
             }
             dB[D1] += dB[0];  // ":698"
             mB[D1] = mB[0];
@@ -380,14 +384,14 @@ void backward_pos(int64_t N, int L, int C, const R* pos, const R* table, const R
 // <q, posgrad(T,g)> = <ggs(q,T), g> = <tablegrad2(q,g), T>.
 
 template <int D, typename R, typename A>
-void double_backward(int64_t N, int L, int C, const R* pos, const R* table, const R* sf, const R* shift,
+void double_backward(int64_t N, int L, int C, int F, const R* pos, const R* table, const R* sf, const R* shift,
                      const R* window, const R* q, const R* grad, R* tgrad, A* tgrad_acc, A* tgrad_abs,
                      R* ggs, A* ggs_abs, int concat_points) {
     constexpr int D1 = D + 1;
-    const int extra = extra_levels(D, concat_points);
+    const int extra = extra_levels(D, F, concat_points);
     for (int l = 0; l < L; ++l) {
         const R w_lvl = window[l];
-        const int64_t base = static_cast<int64_t>(l) * C * 2;
+        const int64_t base = static_cast<int64_t>(l) * C * F;
 #pragma omp parallel for schedule(static)
         for (int64_t n = 0; n < N; ++n) {
             Simplex<D, R> s;
@@ -396,53 +400,42 @@ void double_backward(int64_t N, int L, int C, const R* pos, const R* table, cons
             double_backward_bary<D, R>(s, q + n * D, sf + l * D, dB);
             A mB[D + 2];
             if (ggs_abs) double_backward_bary_magnitude<D, R, A>(s, q + n * D, sf + l * D, mB);
-            A ma0 = 0, ma1 = 0;
-            const R g0 = grad[(static_cast<int64_t>(l) * 2 + 0) * N + n];
-            const R g1 = grad[(static_cast<int64_t>(l) * 2 + 1) * N + n];
-            R gg0 = 0, gg1 = 0;
+            R g[kMaxFeat], gg[kMaxFeat];
+            A ma[kMaxFeat];
+            for (int f = 0; f < F; ++f) {
+                g[f] = grad[(static_cast<int64_t>(l) * F + f) * N + n];
+                gg[f] = 0;
+                ma[f] = 0;
+            }
             for (int r = 0; r <= D; ++r) {
                 int key[D1];
                 vertex_key<D, R>(s, r, key);
-                const int64_t h = base + 2 * static_cast<int64_t>(lattice_slot<D>(key, C));
-                const R t0 = dB[r] * w_lvl * g0, t1 = dB[r] * w_lvl * g1;
-                if (tgrad) {
+                const int64_t h = base + static_cast<int64_t>(F) * lattice_slot<D>(key, C);
+                for (int f = 0; f < F; ++f) {
+                    const R t = dB[r] * w_lvl * g[f];
+                    if (tgrad) {
 #pragma omp atomic
-                    tgrad[h] += t0;
+                        tgrad[h + f] += t;
+                    }
+                    if (tgrad_acc) {
 #pragma omp atomic
-                    tgrad[h + 1] += t1;
-                }
-                if (tgrad_acc) {
+                        tgrad_acc[h + f] += static_cast<A>(t);
+                    }
+                    if (tgrad_abs) {
 #pragma omp atomic
-                    tgrad_acc[h] += static_cast<A>(t0);
-#pragma omp atomic
-                    tgrad_acc[h + 1] += static_cast<A>(t1);
-                }
-                if (tgrad_abs) {
-#pragma omp atomic
-                    tgrad_abs[h] += std::fabs(static_cast<A>(t0));
-#pragma omp atomic
-                    tgrad_abs[h + 1] += std::fabs(static_cast<A>(t1));
-                }
-                if (ggs) {
-                    gg0 += dB[r] * w_lvl * table[h];
-                    gg1 += dB[r] * w_lvl * table[h + 1];
-                }
-                if (ggs_abs) {
-                    ma0 += mB[r] * std::fabs(static_cast<A>(w_lvl)) * std::fabs(static_cast<A>(table[h]));
-                    ma1 += mB[r] * std::fabs(static_cast<A>(w_lvl)) * std::fabs(static_cast<A>(table[h + 1]));
+                        tgrad_abs[h + f] += std::fabs(static_cast<A>(t));
+                    }
+                    if (ggs) gg[f] += dB[r] * w_lvl * table[h + f];
+                    if (ggs_abs) ma[f] += mB[r] * std::fabs(static_cast<A>(w_lvl)) * std::fabs(static_cast<A>(table[h + f]));
                 }
             }
-            if (ggs) {
-                ggs[(static_cast<int64_t>(l) * 2 + 0) * N + n] = gg0;
-                ggs[(static_cast<int64_t>(l) * 2 + 1) * N + n] = gg1;
-            }
-            if (ggs_abs) {
-                ggs_abs[(static_cast<int64_t>(l) * 2 + 0) * N + n] = ma0;
-                ggs_abs[(static_cast<int64_t>(l) * 2 + 1) * N + n] = ma1;
+            for (int f = 0; f < F; ++f) {
+                if (ggs) ggs[(static_cast<int64_t>(l) * F + f) * N + n] = gg[f];
+                if (ggs_abs) ggs_abs[(static_cast<int64_t>(l) * F + f) * N + n] = ma[f];
             }
         }
     }
-    for (int64_t k = static_cast<int64_t>(L) * 2 * N; k < static_cast<int64_t>(L + extra) * 2 * N; ++k) {
+    for (int64_t k = static_cast<int64_t>(L) * F * N; k < static_cast<int64_t>(L + extra) * F * N; ++k) {
         if (ggs) ggs[k] = 0;
         if (ggs_abs) ggs_abs[k] = 0;
     }
@@ -477,6 +470,7 @@ void scale_factors(int D, int L, const float* sigmas, float* sf) {
     }
 
 inline bool bad_sizes(int64_t N, int L, int C) { return N <= 0 || L <= 0 || C <= 0; }
+inline bool bad_feat(int F) { return F < 1 || F > kMaxFeat; }
 
 }  // namespace
 
@@ -517,72 +511,72 @@ int penc_oracle_simplex_f64(int pos_dim, int64_t N, int L, int C, const double* 
     return 0;
 }
 
-int penc_oracle_forward(int pos_dim, int64_t N, int L, int C, const float* pos, const float* table,
+int penc_oracle_forward(int pos_dim, int64_t N, int L, int C, int F, const float* pos, const float* table,
                         const float* sf, const float* shift, const float* window, float* out,
                         int concat_points, float points_scaling) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (forward<DD, float>(N, L, C, pos, table, sf, shift, window, out, concat_points, points_scaling)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (forward<DD, float>(N, L, C, F, pos, table, sf, shift, window, out, concat_points, points_scaling)));
     return 0;
 }
 
-int penc_oracle_forward_f64(int pos_dim, int64_t N, int L, int C, const double* pos, const double* table,
+int penc_oracle_forward_f64(int pos_dim, int64_t N, int L, int C, int F, const double* pos, const double* table,
                             const double* sf, const double* shift, const double* window, double* out,
                             int concat_points, double points_scaling) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (forward<DD, double>(N, L, C, pos, table, sf, shift, window, out, concat_points, points_scaling)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (forward<DD, double>(N, L, C, F, pos, table, sf, shift, window, out, concat_points, points_scaling)));
     return 0;
 }
 
 // tgrad (fp32, omp-atomic), tgrad_acc64 and tgrad_abs64 (fp64 sums of the terms and of their
 // magnitudes) are each optional (NULL) and are accumulated INTO: the caller zero-fills them.
-int penc_oracle_backward_table(int pos_dim, int64_t N, int L, int C, const float* pos, const float* sf,
+int penc_oracle_backward_table(int pos_dim, int64_t N, int L, int C, int F, const float* pos, const float* sf,
                                const float* shift, const float* window, const float* grad,
                                float* tgrad, double* tgrad_acc64, double* tgrad_abs64) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (backward_table<DD, float, double>(N, L, C, pos, sf, shift, window, grad, tgrad, tgrad_acc64, tgrad_abs64)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (backward_table<DD, float, double>(N, L, C, F, pos, sf, shift, window, grad, tgrad, tgrad_acc64, tgrad_abs64)));
     return 0;
 }
 
-int penc_oracle_backward_table_f64(int pos_dim, int64_t N, int L, int C, const double* pos, const double* sf,
+int penc_oracle_backward_table_f64(int pos_dim, int64_t N, int L, int C, int F, const double* pos, const double* sf,
                                    const double* shift, const double* window, const double* grad,
                                    double* tgrad) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (backward_table<DD, double, double>(N, L, C, pos, sf, shift, window, grad, tgrad, nullptr, nullptr)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (backward_table<DD, double, double>(N, L, C, F, pos, sf, shift, window, grad, tgrad, nullptr, nullptr)));
     return 0;
 }
 
-int penc_oracle_backward_pos(int pos_dim, int64_t N, int L, int C, const float* pos, const float* table,
+int penc_oracle_backward_pos(int pos_dim, int64_t N, int L, int C, int F, const float* pos, const float* table,
                              const float* sf, const float* shift, const float* window, const float* grad,
                              float* pgrad, double* pgrad_acc64, double* pgrad_abs64) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (backward_pos<DD, float, double>(N, L, C, pos, table, sf, shift, window, grad, pgrad, pgrad_acc64, pgrad_abs64)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (backward_pos<DD, float, double>(N, L, C, F, pos, table, sf, shift, window, grad, pgrad, pgrad_acc64, pgrad_abs64)));
     return 0;
 }
 
-int penc_oracle_backward_pos_f64(int pos_dim, int64_t N, int L, int C, const double* pos, const double* table,
+int penc_oracle_backward_pos_f64(int pos_dim, int64_t N, int L, int C, int F, const double* pos, const double* table,
                                  const double* sf, const double* shift, const double* window,
                                  const double* grad, double* pgrad) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (backward_pos<DD, double, double>(N, L, C, pos, table, sf, shift, window, grad, pgrad, nullptr, nullptr)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (backward_pos<DD, double, double>(N, L, C, F, pos, table, sf, shift, window, grad, pgrad, nullptr, nullptr)));
     return 0;
 }
 
-int penc_oracle_double_backward(int pos_dim, int64_t N, int L, int C, const float* pos, const float* table,
+int penc_oracle_double_backward(int pos_dim, int64_t N, int L, int C, int F, const float* pos, const float* table,
                                 const float* sf, const float* shift, const float* window,
                                 const float* double_pos_grad, const float* grad, float* tgrad,
                                 double* tgrad_acc64, double* tgrad_abs64, float* ggs, double* ggs_abs64,
                                 int concat_points) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (double_backward<DD, float, double>(N, L, C, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, tgrad_acc64, tgrad_abs64, ggs, ggs_abs64, concat_points)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (double_backward<DD, float, double>(N, L, C, F, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, tgrad_acc64, tgrad_abs64, ggs, ggs_abs64, concat_points)));
     return 0;
 }
 
-int penc_oracle_double_backward_f64(int pos_dim, int64_t N, int L, int C, const double* pos, const double* table,
+int penc_oracle_double_backward_f64(int pos_dim, int64_t N, int L, int C, int F, const double* pos, const double* table,
                                     const double* sf, const double* shift, const double* window,
                                     const double* double_pos_grad, const double* grad, double* tgrad,
                                     double* ggs, int concat_points) {
-    if (bad_sizes(N, L, C)) return 1;
-    DISPATCH_D(pos_dim, (double_backward<DD, double, double>(N, L, C, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, nullptr, nullptr, ggs, nullptr, concat_points)));
+    if (bad_sizes(N, L, C) || bad_feat(F)) return 1;
+    DISPATCH_D(pos_dim, (double_backward<DD, double, double>(N, L, C, F, pos, table, sf, shift, window, double_pos_grad, grad, tgrad, nullptr, nullptr, ggs, nullptr, concat_points)));
     return 0;
 }
 

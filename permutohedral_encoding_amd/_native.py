@@ -36,8 +36,8 @@ _SIGNATURES = {
     "penc_backward_static": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                             _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                             ctypes.c_void_p]),
-    "penc_backward_rowmajor_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
-                                                                 ctypes.c_int, ctypes.c_int]),
+    "penc_backward_rowmajor_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                                                 ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "penc_backward_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                               _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
                                               _c_f32p, _c_f32p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
@@ -112,9 +112,10 @@ def _scatter_bytes(pos_dim, nr_positions, nr_levels, capacity, levels_per_pass):
 
 
 def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device, table_grad=True, positions_grad=False,
-                      fixed_bytes=0, required_bytes=0):
+                      fixed_bytes=0, required_bytes=0, nr_feat=2):
     """Scratch memory for one gradient call (None when the library would not use any).
 
+    The scatter counts every pair of features as a level (``nr_levels * nr_feat / 2`` of them).
     ``fixed_bytes`` is added to every request (the level-major copy of a row-major upstream gradient);
     ``required_bytes`` is the part of it the call cannot do without."""
     if LEVELS_PER_PASS < 0 and not required_bytes:
@@ -122,11 +123,12 @@ def scatter_workspace(pos_dim, nr_positions, nr_levels, capacity, device, table_
     pos_bytes = 0
     if positions_grad:
         pos_bytes = int(lib().penc_positions_workspace_bytes(int(pos_dim), int(nr_positions), int(nr_levels)))
-    per_pass = nr_levels if LEVELS_PER_PASS <= 0 else min(LEVELS_PER_PASS, nr_levels)
+    pair_levels = nr_levels * (nr_feat // 2)
+    per_pass = pair_levels if LEVELS_PER_PASS <= 0 else min(LEVELS_PER_PASS, pair_levels)
     if not table_grad or LEVELS_PER_PASS < 0:
         per_pass = 0
     while True:
-        nbytes = _scatter_bytes(pos_dim, nr_positions, nr_levels, capacity, per_pass) if per_pass else 0
+        nbytes = _scatter_bytes(pos_dim, nr_positions, pair_levels, capacity, per_pass) if per_pass else 0
         nbytes = max(nbytes, pos_bytes) + fixed_bytes
         over_cap = MAX_WORKSPACE_BYTES is not None and nbytes > MAX_WORKSPACE_BYTES
         if not over_cap:
@@ -167,20 +169,20 @@ def _check_f32_gpu(t, name, ndim):
 
 
 def is_row_major_view(grad):
-    """True for a (L, 2, N) *view* of rows grad_rows[n][2*level + feature] (the upstream gradient of the
-    module's (N, 2L) output seen through its permute+reshape): the table gradient can read that as it is."""
+    """True for a (L, F, N) *view* of rows grad_rows[n][F*level + feature] (the upstream gradient of the
+    module's (N, F*L) output seen through its permute+reshape): the library reads that as it is."""
     if grad.dim() != 3 or not grad.is_cuda or grad.dtype != torch.float32 or grad.is_contiguous():
         return False
     levels, feat, n = grad.shape
     s_level, s_feat, s_point = grad.stride()
-    return (feat == 2 and n > 0 and s_level == 2 and s_feat == 1 and s_point >= 2 * levels and s_point % 2 == 0
+    return (feat in (2, 4) and n > 0 and s_level == feat and s_feat == 1 and s_point >= feat * levels and s_point % 2 == 0
             and grad.data_ptr() % 8 == 0 and s_point * n < 2 ** 31)
 
 
 def level_major_gradient(grad):
     """The contiguous (L, 2, N) tensor the gradient kernels read, from whatever autograd hands over.
 
-    The usual case is a (L, 2, N) *view* of a row-major (N, 2L) gradient (what the layer after the
+    The usual case is a (L, F, N) *view* of a row-major (N, F*L) gradient (what the layer after the
     encoding produces, seen through the module's permute+reshape): that is transposed by the
     library at streaming speed.  Anything else takes torch's generic copy (reference: funcs.py:47).
     """
@@ -232,8 +234,8 @@ class EncodingWrapper:
     """The native encoding object (reference: ``EncodingWrapper``, Encoding.cuh:162-188)."""
 
     def __init__(self, pos_dim, nr_feat_per_level, fixed_params):
-        if nr_feat_per_level != 2:
-            raise RuntimeError("Encoding: nr_feat_per_level must be 2 since other values are not yet implemented")
+        if nr_feat_per_level not in (2, 4):
+            raise RuntimeError("Encoding: nr_feat_per_level must be 2 or 4")
         if pos_dim not in (2, 3, 4, 5, 6, 7, 8):
             raise RuntimeError("Encoding: pos_dim must be 2,3,4,5,6,7 or 8")
         self.pos_dim = int(pos_dim)
@@ -255,7 +257,7 @@ class EncodingWrapper:
                  f"with {fp.m_pos_dim} and points have pos dim {pos.shape[1]}")
         _check_f32_gpu(lv, "lattice_values", 3)
         _require(lv.is_contiguous(), "lattice_values must be contiguous (two floats are loaded at a time)")
-        _require(lv.shape[2] == self.nr_feat, "lattice_values should be nr_levels x capacity x 2")
+        _require(lv.shape[2] == self.nr_feat, f"lattice_values should be nr_levels x capacity x {self.nr_feat}")
         levels = lv.shape[0]
         shift = fp.m_random_shift_per_level
         _check_f32_gpu(shift, "random_shift_per_level", 2)
@@ -311,15 +313,16 @@ class EncodingWrapper:
             return None, None
         with torch.cuda.device(pos.device):
             if not grad.is_contiguous():  # rows (N, 2(L+E))
-                copy_bytes = 8 * levels * n + 512 if pos_grad is not None else 0
+                copy_bytes = 4 * self.nr_feat * levels * n + 512 if pos_grad is not None else 0
                 ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None,
-                                       fixed_bytes=copy_bytes, required_bytes=copy_bytes)
+                                       fixed_bytes=copy_bytes, required_bytes=copy_bytes, nr_feat=self.nr_feat)
                 _check(lib().penc_backward_rowmajor(
                     self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
                     _ptr(win), _ptr(grad), grad.stride(2), _ptr(lv_grad), _ptr(pos_grad), _ptr(ws),
                     0 if ws is None else ws.numel(), _stream()), "backward")
                 return lv_grad, pos_grad
-            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None)
+            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None,
+                                   nr_feat=self.nr_feat)
             _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
                                        _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(grad), _ptr(lv_grad),
                                        _ptr(pos_grad), _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
@@ -341,7 +344,7 @@ class EncodingWrapper:
         lv_grad = torch.empty_like(lv)
         ggs = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
         with torch.cuda.device(pos.device):
-            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device)
+            ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, nr_feat=self.nr_feat)
             if not grad.is_contiguous():
                 _check(lib().penc_double_backward_from_positions_rowmajor(
                     self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),

@@ -32,10 +32,6 @@ constexpr int pos_levels_per_group(int pos_dim) { return pos_dim >= 6 ? 1 : 2; }
 
 constexpr int kDefaultLevelsPerPass = 1 << 20;  // by default the suggested workspace bins all levels in one pass (measured fastest)
 
-__device__ __forceinline__ float2 load_vertex(const float* __restrict__ level_table, uint32_t slot) {
-    return *reinterpret_cast<const float2*>(level_table + 2 * static_cast<size_t>(slot));
-}
-
 template <int D>
 __device__ __forceinline__ fvec<D> load_point(const float* __restrict__ positions, int64_t n) {
     const float* p = positions + n * D;
@@ -45,20 +41,31 @@ __device__ __forceinline__ fvec<D> load_point(const float* __restrict__ position
     return pos;
 }
 
-// The D+1 table entries of a simplex, fetched back to back so that all loads are in flight together.
-template <int D>
+// The D+1 table entries of a simplex (F features each: one 8- or 16-byte load per vertex), fetched
+// back to back so that all loads are in flight together.  f[k][r] is feature k of vertex r.
+template <int D, int F>
 struct Vertices {
-    fvec<D + 1> f0, f1;
+    fvec<D + 1> f[F];
 };
-template <int D>
-__device__ __forceinline__ Vertices<D> load_vertices(const float* __restrict__ level_table, uvec<D + 1> h,
-                                                     uint32_t capacity, uint32_t cap_mask) {
-    Vertices<D> v;
+template <int D, int F>
+__device__ __forceinline__ Vertices<D, F> load_vertices(const float* __restrict__ level_table, uvec<D + 1> h,
+                                                        uint32_t capacity, uint32_t cap_mask) {
+    static_assert(F == 2 || F == 4, "two or four features per level");
+    Vertices<D, F> v;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
-        const float2 x = load_vertex(level_table, to_slot(h[r], capacity, cap_mask));
-        v.f0[r] = x.x;
-        v.f1[r] = x.y;
+        const size_t slot = to_slot(h[r], capacity, cap_mask);
+        if constexpr (F == 2) {
+            const float2 x = *reinterpret_cast<const float2*>(level_table + 2 * slot);
+            v.f[0][r] = x.x;
+            v.f[1][r] = x.y;
+        } else {
+            const float4 x = *reinterpret_cast<const float4*>(level_table + 4 * slot);
+            v.f[0][r] = x.x;
+            v.f[1][r] = x.y;
+            v.f[2][r] = x.z;
+            v.f[3][r] = x.w;
+        }
     });
     return v;
 }
@@ -74,7 +81,7 @@ __device__ __forceinline__ Vertices<D> load_vertices(const float* __restrict__ l
 // (compute-bound) and a fine (gather-bound) level, which takes the fine level's slice out of L2
 // (30% slower).
 
-template <int D>
+template <int D, int F>
 __global__ void __launch_bounds__(kBlock)
 forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
                const float* __restrict__ positions, const float* __restrict__ table,
@@ -83,20 +90,21 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
     const int n = blockIdx.x * kBlock + threadIdx.x;
     if (n >= n_points) return;
     const int level = blockIdx.y;
-    float* out0 = sliced + (static_cast<size_t>(level) * 2) * n_points + n;
-    float* out1 = out0 + n_points;
+    float* out = sliced + (static_cast<size_t>(level) * F) * n_points + n;  // feature k at out[k * n_points]
 
     if (level >= n_levels) {  // extra levels carrying the raw positions (:106-121)
-        const int src = (level - n_levels) * 2;
+        const int src = (level - n_levels) * F;
         const float* p = positions + static_cast<size_t>(n) * D;
-        *out0 = src < D ? p[src] * points_scaling : 0.0f;
-        *out1 = src + 1 < D ? p[src + 1] * points_scaling : 0.0f;
+        static_for<F>(PENC_BODY(k) {
+            PENC_INDEX(k);
+            out[static_cast<size_t>(k) * n_points] = src + k < D ? p[src + k] * points_scaling : 0.0f;
+        });
         return;
     }
     const float w_level = window[level];
     if (w_level == 0.0f) {
-        *out0 = 0.0f;
-        *out1 = 0.0f;
+        static_for<F>(PENC_BODY(k) {
+            PENC_INDEX(k); out[static_cast<size_t>(k) * n_points] = 0.0f; });
         return;
     }
     const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, scale_factor + level * D);
@@ -107,16 +115,16 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
     fvec<D + 1> sorted;
     sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, s.delta, s.hash0, sorted, h);
     const fvec<D + 1> w = barycentric_of_sorted<D>(sorted);
-    const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
-    float acc0 = 0.0f, acc1 = 0.0f;
+    const Vertices<D, F> v = load_vertices<D, F>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+    fvec<F> acc = 0.0f;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
         const float wr = w[r] * w_level;
-        acc0 = acc0 + v.f0[r] * wr;
-        acc1 = acc1 + v.f1[r] * wr;
+        static_for<F>(PENC_BODY(k) {
+            PENC_INDEX(k); acc[k] = acc[k] + v.f[k][r] * wr; });
     });
-    *out0 = acc0;
-    *out1 = acc1;
+    static_for<F>(PENC_BODY(k) {
+        PENC_INDEX(k); out[static_cast<size_t>(k) * n_points] = acc[k]; });
 }
 
 // ------------------------------------------------------------------------------------------
@@ -132,10 +140,14 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 // kSecondOrder: the table-gradient half of the double backward (EncodingGPU.cuh:1016-1257): the
 // vertex weights are the derivatives of the barycentric weights along `double_pos_grad` instead of
 // the barycentric weights themselves; everything else is the same scatter.
+// feat_pairs: with four features per level the pairs (0,1) and (2,3) are scattered like two levels that
+// share their geometry: "levels" below (first_level, n_pass_levels, the grid, the bins) count pairs,
+// `pair_level` = level * feat_pairs + pair.  The upstream gradient needs no special case: [L][F][N]
+// is [L * F/2][2][N], and in a row the pair sits at column 2 * pair_level.
 template <int D, bool kRowMajor, bool kSecondOrder>
 __global__ void __launch_bounds__(kScatterBlock)
-backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int tiles_per_group, uint32_t capacity,
-                      uint32_t cap_mask,
+backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t feat_pairs, int tiles_per_group,
+                      uint32_t capacity, uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
                       const float* __restrict__ grad_sliced, int64_t grad_row_stride,
@@ -152,20 +164,22 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
     const uint32_t level_in_pass = j % n_pass_levels, group = (j / n_pass_levels) * kXcds + die;
     const int64_t group_base = static_cast<int64_t>(group) * tiles_per_group * kScatterBlock;
     if (group_base >= n_points) return;
-    const int level = first_level + level_in_pass;
+    const uint32_t pair_level = static_cast<uint32_t>(first_level) + level_in_pass;
+    const int level = static_cast<int>(pair_level / feat_pairs);  // the geometry's level
     const float w_level = window[level];
     if (w_level == 0.0f) return;
     scatter_begin(state);
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
-    float* level_grad = table_grad + static_cast<size_t>(level) * capacity * 2;
+    const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair_level % feat_pairs) * 2,
+                               2 * feat_pairs};
     // Everything a thread reads lies within its group of at most 16 x 512 points, so the addresses are
     // wave-uniform 64-bit bases (scalar registers) plus 32-bit per-thread offsets.
     const uint32_t last_in_group = static_cast<uint32_t>(n_points - 1 - group_base);
     const float* const group_positions = positions + group_base * D;
     const float* const group_q = kSecondOrder ? double_pos_grad + group_base * D : nullptr;
     const float* const group_grad0 =
-        kRowMajor ? grad_sliced + group_base * grad_row_stride + 2 * level
-                  : grad_sliced + (static_cast<size_t>(level) * 2) * n_points + group_base;
+        kRowMajor ? grad_sliced + group_base * grad_row_stride + 2 * pair_level
+                  : grad_sliced + (static_cast<size_t>(pair_level) * 2) * n_points + group_base;
     const float* const group_grad1 = group_grad0 + n_points;
     const auto load_grad = [&](uint32_t i, float& g0, float& g1) {
         if constexpr (kRowMajor) {
@@ -208,7 +222,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
         load_grad(nn_next, g0_next, g1_next);
         if constexpr (kRowMajor) {
             if (grad_level_major != nullptr && active) {
-                float* out = grad_level_major + (static_cast<size_t>(level) * 2) * n_points + tile_base + threadIdx.x;
+                float* out = grad_level_major + (static_cast<size_t>(pair_level) * 2) * n_points + tile_base + threadIdx.x;
                 out[0] = g0;
                 out[n_points] = g1;
             }
@@ -248,7 +262,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, int
 // the whole chip on the same few levels at a time (their table slices stay in L2) and give the
 // launch many more, shorter waves than one thread per point walking all levels.  (Doing this
 // kernel's rank permutations through LDS, as the forward does, was measured: no gain.)
-template <int D>
+template <int D, int F>
 __global__ void __launch_bounds__(kBlock)
 backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t capacity, uint32_t cap_mask,
                     const float* __restrict__ positions, const float* __restrict__ table,
@@ -267,10 +281,14 @@ backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t c
         const float* sf = scale_factor + level * D;
         const Located<D> s = locate<D>(pos, random_shift + level * D, sf);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
-        const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
-        const float* gp = grad_sliced + (static_cast<size_t>(level) * 2) * n_points + n;
-        const float g0 = gp[0], g1 = gp[n_points];
-        const fvec<D + 1> dB = (v.f0 * w_level) * g0 + (v.f1 * w_level) * g1;  // :688-689
+        const Vertices<D, F> v = load_vertices<D, F>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+        const float* gp = grad_sliced + (static_cast<size_t>(level) * F) * n_points + n;
+        fvec<D + 1> dB = (v.f[0] * w_level) * gp[0];  // :688-689, feature by feature
+        static_for<F - 1>(PENC_BODY(kk) {
+            PENC_INDEX(kk);
+            constexpr int k = kk + 1;
+            dB += (v.f[k] * w_level) * gp[static_cast<size_t>(k) * n_points];
+        });
         total += bary_grad_to_pos_grad<D>(s.rank, dB, sf);
     }
     float* o = out + (static_cast<size_t>(blockIdx.y) * n_points + n) * D;
@@ -298,7 +316,7 @@ reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size
 // was measured 7-13% slower than the two: the gathering half wants small workgroups, the scattering
 // half large groups of points with the levels interleaved.)
 
-template <int D>
+template <int D, int F>
 __global__ void __launch_bounds__(kBlock)
 grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
                  const float* __restrict__ positions, const float* __restrict__ table,
@@ -308,11 +326,11 @@ grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mas
     const int n = blockIdx.x * kBlock + threadIdx.x;
     if (n >= n_points) return;
     const int level = blockIdx.y;
-    float* o = grad_grad_sliced + (static_cast<size_t>(level) * 2) * n_points + n;
+    float* o = grad_grad_sliced + (static_cast<size_t>(level) * F) * n_points + n;
     const float w_level = level < n_levels ? window[level] : 0.0f;  // concat levels: zeros (:1290-1295)
     if (w_level == 0.0f) {
-        o[0] = 0.0f;
-        o[n_points] = 0.0f;
+        static_for<F>(PENC_BODY(k) {
+            PENC_INDEX(k); o[static_cast<size_t>(k) * n_points] = 0.0f; });
         return;
     }
     const float* sf = scale_factor + level * D;
@@ -324,17 +342,17 @@ grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mas
     fvec<D + 1> sorted;
     sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, pos_grad_grad_to_elevated<D>(load_point<D>(double_pos_grad, n), sf),
                         s.hash0, sorted, h);
-    const Vertices<D> v = load_vertices<D>(table + static_cast<size_t>(level) * capacity * 2, h, capacity, cap_mask);
+    const Vertices<D, F> v = load_vertices<D, F>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
     // dB[r] * w_level, then times the vertex value (:1484-1485)
     const fvec<D + 1> wr = sorted_elevated_grad_to_bary<D>(sorted) * w_level;
-    float gg0 = 0.0f, gg1 = 0.0f;
+    fvec<F> gg = 0.0f;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
-        gg0 += wr[r] * v.f0[r];
-        gg1 += wr[r] * v.f1[r];
+        static_for<F>(PENC_BODY(k) {
+            PENC_INDEX(k); gg[k] += wr[r] * v.f[k][r]; });
     });
-    o[0] = gg0;
-    o[n_points] = gg1;
+    static_for<F>(PENC_BODY(k) {
+        PENC_INDEX(k); o[static_cast<size_t>(k) * n_points] = gg[k]; });
 }
 
 // ------------------------------------------------------------------------------------------
@@ -432,22 +450,24 @@ inline uint32_t mask_of(int capacity) {
 
 inline int check_geometry(int pos_dim, int nr_feat, int64_t n, int levels, int capacity, int extra) {
     if (pos_dim < 2 || pos_dim > 8) return PENC_ERR_UNSUPPORTED_POS_DIM;
-    if (nr_feat != 2) return PENC_ERR_UNSUPPORTED_NR_FEAT;
+    if (nr_feat != 2 && nr_feat != 4) return PENC_ERR_UNSUPPORTED_NR_FEAT;
     if (n <= 0 || levels <= 0 || capacity <= 0) return PENC_ERR_BAD_SIZE;
     const int64_t lim = (int64_t{1} << 31) - 1;
-    if (n > lim / (2 * (int64_t{levels} + extra)) || n > lim / pos_dim) return PENC_ERR_BAD_SIZE;
-    if (int64_t{capacity} > lim / (2 * int64_t{levels})) return PENC_ERR_BAD_SIZE;
+    if (n > lim / (nr_feat * (int64_t{levels} + extra)) || n > lim / pos_dim) return PENC_ERR_BAD_SIZE;
+    if (int64_t{capacity} > lim / (nr_feat * int64_t{levels})) return PENC_ERR_BAD_SIZE;
     if (levels + extra > 65535) return PENC_ERR_BAD_SIZE;
     return PENC_OK;
 }
 
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+// the table is gathered with one load per slot: 8 bytes for two features, 16 for four
+inline bool table_aligned(const void* p, int nr_feat) { return (reinterpret_cast<uintptr_t>(p) & (nr_feat == 4 ? 15u : 7u)) == 0; }
 
 // Clears the table gradient with a fill kernel (float2 granularity: the array is only guaranteed
 // 8-byte alignment).  A kernel rather than hipMemsetAsync so that callers may capture the call in
 // a HIP graph.
-inline int clear_table_grad(float* g, int levels, int capacity, hipStream_t st) {
-    const size_t n2 = static_cast<size_t>(levels) * capacity;
+inline int clear_table_grad(float* g, int pair_levels, int capacity, hipStream_t st) {
+    const size_t n2 = static_cast<size_t>(pair_levels) * capacity;
     const size_t want = (n2 + kBlock * 8 - 1) / (kBlock * 8);
     const unsigned blocks = static_cast<unsigned>(want < 8192 ? want : 8192);
     hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(kBlock), 0, st, reinterpret_cast<float2*>(g), n2);
@@ -541,14 +561,14 @@ constexpr unsigned kReduceWorkgroupsWanted = 512;  // two per compute unit
 constexpr unsigned kMaxReduceSplits = 16;
 
 inline int reduce_bins(const BinPlan& p, const float* window, int first_level, int n_levels_in_pass, int capacity,
-                       float* table_grad, hipStream_t st) {
+                       uint32_t feat_pairs, float* table_grad, hipStream_t st) {
     // enough workgroups for every compute unit, by letting several share a bin when bins*levels is small
     const unsigned pairs = p.target.n_bins * static_cast<unsigned>(n_levels_in_pass);
     unsigned splits = pairs >= kReduceWorkgroupsWanted ? 1u : (kReduceWorkgroupsWanted + pairs - 1) / pairs;
     if (splits > p.target.n_groups) splits = p.target.n_groups;
     if (splits > kMaxReduceSplits) splits = kMaxReduceSplits;
     hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass, splits), dim3(kReduceBlock), 0, st,
-                       p.target, window, static_cast<uint32_t>(capacity), table_grad, first_level);
+                       p.target, window, static_cast<uint32_t>(capacity), feat_pairs, table_grad, first_level);
     return check_launch();
 }
 
@@ -562,6 +582,16 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
         case 7: { constexpr int DD = 7; __VA_ARGS__; } break;      \
         case 8: { constexpr int DD = 8; __VA_ARGS__; } break;      \
         default: return PENC_ERR_UNSUPPORTED_POS_DIM;              \
+    }
+
+// The same with the number of features per level (2 or 4) as the constant FF.
+#define PENC_DISPATCH_DF(D_, F_, ...)                                   \
+    if ((F_) == 4) {                                                    \
+        constexpr int FF = 4;                                           \
+        PENC_DISPATCH_D(D_, __VA_ARGS__)                                \
+    } else {                                                            \
+        constexpr int FF = 2;                                           \
+        PENC_DISPATCH_D(D_, __VA_ARGS__)                                \
     }
 
 inline unsigned tiles(int64_t n) { return static_cast<unsigned>((n + kBlock - 1) / kBlock); }
@@ -595,27 +625,30 @@ using namespace penc;
 // the [level][feature][n] layout, otherwise the gradient is rows of that many floats.  With
 // double_pos_grad the same for the table-gradient half of the double backward.  grad_level_major (rows
 // only, may be NULL) receives the upstream gradient in [level][feature][n] order as a by-product.
-static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
+static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
                           const float* scale_factor, const float* random_shift, const float* anneal_window,
                           const float* grad, int64_t grad_row_stride, const float* double_pos_grad,
                           float* lattice_values_grad, float* grad_level_major, void* workspace, size_t workspace_bytes,
                           hipStream_t st) {
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
-    if (int rc = clear_table_grad(lattice_values_grad, nr_levels, capacity, st)) return rc;
-    const int tiles_per_group = table_backward_tiles(nr_positions, nr_levels);
-    const BinPlan plan = plan_bins(pos_dim, nr_positions, nr_levels, capacity, tiles_per_group, workspace, workspace_bytes);
-    const int per_pass = plan.enabled ? plan.levels_per_pass : nr_levels;
-    for (int first = 0; first < nr_levels; first += per_pass) {
-        const int count = nr_levels - first < per_pass ? nr_levels - first : per_pass;
+    // every pair of features is scattered like a level of its own (see backward_table_kernel)
+    const uint32_t feat_pairs = static_cast<uint32_t>(nr_feat / 2);
+    const int pair_levels = nr_levels * static_cast<int>(feat_pairs);
+    if (int rc = clear_table_grad(lattice_values_grad, pair_levels, capacity, st)) return rc;
+    const int tiles_per_group = table_backward_tiles(nr_positions, pair_levels);
+    const BinPlan plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
+    const int per_pass = plan.enabled ? plan.levels_per_pass : pair_levels;
+    for (int first = 0; first < pair_levels; first += per_pass) {
+        const int count = pair_levels - first < per_pass ? pair_levels - first : per_pass;
         const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
         const dim3 grid(padded_groups * static_cast<unsigned>(count));
 #define PENC_LAUNCH_TABLE(ROW_MAJOR, SECOND_ORDER)                                                                         \
     PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER>), grid,                  \
                                                 dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
-                                                tiles_per_group, cap, mask, positions, scale_factor, random_shift,           \
-                                                anneal_window, grad, grad_row_stride, double_pos_grad, lattice_values_grad,  \
-                                                grad_level_major, plan.target))
+                                                feat_pairs, tiles_per_group, cap, mask, positions, scale_factor,             \
+                                                random_shift, anneal_window, grad, grad_row_stride, double_pos_grad,         \
+                                                lattice_values_grad, grad_level_major, plan.target))
         if (double_pos_grad != nullptr && grad_row_stride != 0) {
             PENC_LAUNCH_TABLE(true, true);
         } else if (double_pos_grad != nullptr) {
@@ -628,7 +661,7 @@ static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int 
 #undef PENC_LAUNCH_TABLE
         if (int rc = check_launch()) return rc;
         if (plan.enabled)
-            if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, lattice_values_grad, st)) return rc;
+            if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, feat_pairs, lattice_values_grad, st)) return rc;
     }
     return PENC_OK;
 }
@@ -636,7 +669,7 @@ static int table_backward(int pos_dim, int64_t nr_positions, int nr_levels, int 
 // The position gradient of penc_backward / penc_backward_rowmajor from a level-major upstream gradient:
 // levels in groups of pos_levels_per_group() when the workspace can hold the partial sums, else one
 // thread per point walks all levels.
-static int positions_backward(int pos_dim, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
+static int positions_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
                               const float* lattice_values, const float* scale_factor, const float* random_shift,
                               const float* anneal_window, const float* grad_level_major, float* positions_grad,
                               void* workspace, size_t workspace_bytes, hipStream_t st) {
@@ -653,10 +686,10 @@ static int positions_backward(int pos_dim, int64_t nr_positions, int nr_levels, 
         groups = want_groups;
         partial = reinterpret_cast<float*>(ws);
     }
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_pos_kernel<DD>), dim3(tiles(nr_positions), groups),
-                                                dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
-                                                lattice_values, scale_factor, random_shift, anneal_window,
-                                                grad_level_major, partial));
+    PENC_DISPATCH_DF(pos_dim, nr_feat, hipLaunchKernelGGL((backward_pos_kernel<DD, FF>), dim3(tiles(nr_positions), groups),
+                                                         dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
+                                                         lattice_values, scale_factor, random_shift, anneal_window,
+                                                         grad_level_major, partial));
     if (int rc = check_launch()) return rc;
     if (groups > 1) {
         const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
@@ -687,15 +720,15 @@ static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
         return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
     if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
-    if ((lattice_values && !aligned8(lattice_values)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    if ((lattice_values && !table_aligned(lattice_values, nr_feat)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (lattice_values_grad)
-        if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+        if (int rc = table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
                                     anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, nullptr, workspace,
                                     workspace_bytes, st))
             return rc;
     if (positions_grad)
-        return positions_backward(pos_dim, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+        return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
                                   random_shift, anneal_window, grad_sliced_values, positions_grad, workspace, workspace_bytes, st);
     return PENC_OK;
 }
@@ -708,8 +741,8 @@ const char* penc_status_string(int status) {
         case PENC_ERR_NULL_POINTER: return "a required pointer is NULL";
         case PENC_ERR_BAD_SIZE: return "nr_positions, nr_levels and capacity must be positive and every array must stay below 2^31 elements";
         case PENC_ERR_UNSUPPORTED_POS_DIM: return "pos_dim must be 2,3,4,5,6,7 or 8";
-        case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2 since other values are not implemented";
-        case PENC_ERR_MISALIGNED: return "lattice_values and lattice_values_grad must be 8-byte aligned";
+        case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2 or 4";
+        case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to one slot (8 bytes for two features, 16 for four), lattice_values_grad and gradient rows to 8 bytes";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
         case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major copy of the upstream gradient (penc_backward_rowmajor_workspace_bytes)";
         case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
@@ -767,14 +800,14 @@ int penc_forward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, 
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
     if (!positions || !lattice_values || !scale_factor || !random_shift || !anneal_window || !sliced_values)
         return PENC_ERR_NULL_POINTER;
-    if (!aligned8(lattice_values)) return PENC_ERR_MISALIGNED;
+    if (!table_aligned(lattice_values, nr_feat)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid(tiles(nr_positions), nr_levels + extra);
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((forward_kernel<DD>), grid, dim3(kBlock), 0, st,
-                                                static_cast<int>(nr_positions), nr_levels,
-                                                static_cast<uint32_t>(capacity), mask_of(capacity), positions,
-                                                lattice_values, scale_factor, random_shift, anneal_window,
-                                                sliced_values, points_scaling));
+    PENC_DISPATCH_DF(pos_dim, nr_feat, hipLaunchKernelGGL((forward_kernel<DD, FF>), grid, dim3(kBlock), 0, st,
+                                                         static_cast<int>(nr_positions), nr_levels,
+                                                         static_cast<uint32_t>(capacity), mask_of(capacity), positions,
+                                                         lattice_values, scale_factor, random_shift, anneal_window,
+                                                         sliced_values, points_scaling));
     return check_launch();
 }
 
@@ -808,23 +841,25 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                          PENC_STATIC_SCRATCH_BYTES, stream);
 }
 
-static int check_rows(const float* grad_rows, int64_t grad_row_stride, int64_t nr_positions, int nr_levels) {
+static int check_rows(const float* grad_rows, int64_t grad_row_stride, int64_t nr_positions, int nr_levels, int nr_feat) {
     if (!grad_rows) return PENC_ERR_NULL_POINTER;
-    if (grad_row_stride < 2 * static_cast<int64_t>(nr_levels) || (grad_row_stride & 1) != 0 ||
+    if (grad_row_stride < nr_feat * static_cast<int64_t>(nr_levels) || (grad_row_stride & 1) != 0 ||
         grad_row_stride * nr_positions >= (int64_t{1} << 31))
         return PENC_ERR_BAD_SIZE;
     if (!aligned8(grad_rows)) return PENC_ERR_MISALIGNED;
     return PENC_OK;
 }
 
-size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels, int capacity,
+size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
                                               int want_lattice_values_grad, int want_positions_grad) {
-    if (pos_dim < 2 || pos_dim > 8 || nr_positions <= 0 || nr_levels <= 0 || capacity <= 0) return 0;
+    if (pos_dim < 2 || pos_dim > 8 || (nr_feat != 2 && nr_feat != 4) || nr_positions <= 0 || nr_levels <= 0 || capacity <= 0)
+        return 0;
     size_t scratch = 0;
-    if (want_lattice_values_grad) scratch = penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels, capacity, 0);
+    if (want_lattice_values_grad)
+        scratch = penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels * (nr_feat / 2), capacity, 0);
     if (!want_positions_grad) return scratch;
     const size_t partial = penc_positions_workspace_bytes(pos_dim, nr_positions, nr_levels);
-    const size_t copy = static_cast<size_t>(nr_levels) * 2 * static_cast<size_t>(nr_positions) * sizeof(float);
+    const size_t copy = static_cast<size_t>(nr_levels) * nr_feat * static_cast<size_t>(nr_positions) * sizeof(float);
     return 512 + copy + (scratch > partial ? scratch : partial);
 }
 
@@ -837,16 +872,16 @@ int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int n
     if (!positions || !scale_factor || !random_shift || !anneal_window) return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
     if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
-    if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels)) return rc;
-    if ((lattice_values && !aligned8(lattice_values)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
+    if ((lattice_values && !table_aligned(lattice_values, nr_feat)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (!positions_grad)
-        return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+        return table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
                               anneal_window, grad_rows, grad_row_stride, nullptr, lattice_values_grad, nullptr, workspace,
                               workspace_bytes, st);
     // The position gradient gathers level by level and reads its upstream gradient as [level][feature][n]:
     // that copy lives at the front of the workspace; the rest serves the scatter and then the partial sums.
-    const size_t copy_bytes = static_cast<size_t>(nr_levels) * 2 * static_cast<size_t>(nr_positions) * sizeof(float);
+    const size_t copy_bytes = static_cast<size_t>(nr_levels) * nr_feat * static_cast<size_t>(nr_positions) * sizeof(float);
     const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
     const size_t lost = base - reinterpret_cast<uintptr_t>(workspace);
     if (workspace == nullptr || workspace_bytes < lost + copy_bytes) return PENC_ERR_WORKSPACE_TOO_SMALL;
@@ -856,16 +891,16 @@ int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int n
     const size_t rest_bytes = rest ? workspace_bytes - lost - copy_span : 0;
     if (lattice_values_grad) {
         // the scattering kernel reads every (point, level) pair of the rows anyway and leaves the copy behind
-        if (int rc = table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
+        if (int rc = table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
                                     anneal_window, grad_rows, grad_row_stride, nullptr, lattice_values_grad, level_major,
                                     rest, rest_bytes, st))
             return rc;
     } else {
-        const int cols = 2 * nr_levels;
+        const int cols = nr_feat * nr_levels;
         if (cols > 255) return PENC_ERR_BAD_SIZE;
         if (int rc = transpose_rows(grad_rows, grad_row_stride, level_major, nr_positions, cols, st)) return rc;
     }
-    return positions_backward(pos_dim, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+    return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
                               random_shift, anneal_window, level_major, positions_grad, rest, rest_bytes, st);
 }
 
@@ -891,19 +926,19 @@ static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, 
         !double_positions_grad || !grad)
         return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !grad_grad_sliced_values) return PENC_ERR_NULL_POINTER;
-    if (!aligned8(lattice_values) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    if (!table_aligned(lattice_values, nr_feat) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (grad_grad_sliced_values) {
         const dim3 grid(tiles(nr_positions), nr_levels + extra);
-        PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((grad_grad_kernel<DD>), grid, dim3(kBlock), 0, st,
-                                                    static_cast<int>(nr_positions), nr_levels,
-                                                    static_cast<uint32_t>(capacity), mask_of(capacity), positions,
-                                                    lattice_values, scale_factor, random_shift, anneal_window,
-                                                    double_positions_grad, grad_grad_sliced_values));
+        PENC_DISPATCH_DF(pos_dim, nr_feat, hipLaunchKernelGGL((grad_grad_kernel<DD, FF>), grid, dim3(kBlock), 0, st,
+                                                             static_cast<int>(nr_positions), nr_levels,
+                                                             static_cast<uint32_t>(capacity), mask_of(capacity), positions,
+                                                             lattice_values, scale_factor, random_shift, anneal_window,
+                                                             double_positions_grad, grad_grad_sliced_values));
         if (int rc = check_launch()) return rc;
     }
     if (!lattice_values_grad) return PENC_OK;
-    return table_backward(pos_dim, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
+    return table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
                           grad, grad_row_stride, double_positions_grad, lattice_values_grad, nullptr, workspace,
                           workspace_bytes, st);
 }
@@ -931,7 +966,7 @@ int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64
                                                  int concat_points, void* workspace, size_t workspace_bytes,
                                                  void* stream) {
     if (nr_levels > 0 && nr_positions > 0)
-        if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels)) return rc;
+        if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
     return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values,
                                 scale_factor, random_shift, anneal_window, double_positions_grad, grad_rows,
                                 grad_row_stride, lattice_values_grad, grad_grad_sliced_values, concat_points, workspace,

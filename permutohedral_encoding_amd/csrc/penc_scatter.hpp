@@ -83,6 +83,15 @@ __device__ __forceinline__ BinTarget bins_of_level(const BinTarget& pass, uint32
     return t;
 }
 
+// One level's slice of the table gradient as the scatter sees it: a pair of features per slot,
+// `slot_floats` floats from one slot to the next (2 when a level has two features; with four, the
+// slice of features (0,1) or (2,3) of an array whose slots are four floats apart).
+struct GradSlice {
+    float* base;
+    uint32_t slot_floats;
+    __device__ __forceinline__ float* at(uint32_t slot) const { return base + static_cast<size_t>(slot) * slot_floats; }
+};
+
 __device__ __forceinline__ void global_add(float* addr, float v) {
     __hip_atomic_fetch_add(addr, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -134,7 +143,7 @@ __device__ __forceinline__ void wave_lds_fence() {
 // Stage 3.  Lanes are paired (2p, 2p+1): first both lanes of a pair add the two features of the
 // even lane's slot, then those of the odd lane's slot, so that each 8-byte slot is one request.
 // Must be called with all 64 lanes of the wave active.
-__device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad, bool need, uint32_t slot,
+__device__ __forceinline__ void global_add_pairs(const GradSlice& level_grad, bool need, uint32_t slot,
                                                  float a0, float a1) {
     constexpr int kFromEven = 0xA0;  // quad_perm:[0,0,2,2]
     constexpr int kFromOdd = 0xF5;   // quad_perm:[1,1,3,3]
@@ -146,14 +155,14 @@ __device__ __forceinline__ void global_add_pairs(float* __restrict__ level_grad,
         const int n = __builtin_amdgcn_update_dpp(0, need_i, kFromEven, 0xf, 0xf, true);
         const int hi = __builtin_amdgcn_update_dpp(0, a1_i, kFromEven, 0xf, 0xf, true);
         const float v = __builtin_bit_cast(float, odd ? hi : a0_i);
-        if (n) global_add(level_grad + 2 * static_cast<size_t>(static_cast<uint32_t>(s)) + odd, v);
+        if (n) global_add(level_grad.at(static_cast<uint32_t>(s)) + odd, v);
     }
     {   // the odd lane's contribution
         const int s = __builtin_amdgcn_update_dpp(0, slot_i, kFromOdd, 0xf, 0xf, true);
         const int n = __builtin_amdgcn_update_dpp(0, need_i, kFromOdd, 0xf, 0xf, true);
         const int lo = __builtin_amdgcn_update_dpp(0, a0_i, kFromOdd, 0xf, 0xf, true);
         const float v = __builtin_bit_cast(float, odd ? a1_i : lo);
-        if (n) global_add(level_grad + 2 * static_cast<size_t>(static_cast<uint32_t>(s)) + odd, v);
+        if (n) global_add(level_grad.at(static_cast<uint32_t>(s)) + odd, v);
     }
 }
 
@@ -235,7 +244,7 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
 // Needs bins.n_bins <= kStageBins and a level's record array below 2^32 bytes (the host plans
 // for both); all 64 lanes of the wave must call it together.
 template <int D>
-__device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+__device__ __forceinline__ void stream_tile(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
                                             fvec<D + 1> a1) {
     constexpr int kWaves = kScatterBlock / 64;
@@ -348,7 +357,7 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, float* __restrict__
 // has seen that the cache does not hit at this level; `streaming` is what scatter_stream_switch
 // returned.  The return value is the number of hits of this wave in this tile.
 template <int D>
-__device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+__device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
                                                  uint32_t group, bool active, bool use_cache, bool streaming,
                                                  uvec<D + 1> slot, fvec<D + 1> a0, fvec<D + 1> a1) {
     if (streaming) {
@@ -409,7 +418,7 @@ __device__ __forceinline__ bool cache_pays(const ScatterState& c, int tiles_done
 }
 
 // Sends every line of the accumulate cache on to stage 2 (or 3).  By all threads, between barriers.
-__device__ __forceinline__ void cache_flush(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+__device__ __forceinline__ void cache_flush(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group) {
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         const int owner = c.tag[e];
@@ -417,7 +426,7 @@ __device__ __forceinline__ void cache_flush(ScatterState& c, float* __restrict__
             const float v0 = static_cast<float>(c.val[0][e]), v1 = static_cast<float>(c.val[1][e]);
             const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
             if (!binned) {
-                float* g = level_grad + 2 * static_cast<size_t>(owner);
+                float* g = level_grad.at(static_cast<uint32_t>(owner));
                 global_add(g, v0);
                 global_add(g + 1, v1);
             }
@@ -429,7 +438,7 @@ __device__ __forceinline__ void cache_flush(ScatterState& c, float* __restrict__
 // workgroup whether to give up the accumulate cache for good and use its LDS as staging space
 // (stream_tile).  Returns true from then on; the cache's contents have been flushed by then.
 template <int D>
-__device__ __forceinline__ bool scatter_stream_switch(ScatterState& c, float* __restrict__ level_grad,
+__device__ __forceinline__ bool scatter_stream_switch(ScatterState& c, const GradSlice& level_grad,
                                                       const BinTarget& bins, uint32_t group, int tile) {
     if (tile != kStreamDecisionTile || bins.records == nullptr || bins.n_bins > kStageBins) return false;
     __syncthreads();  // the hits of the tiles so far are in
@@ -444,7 +453,7 @@ __device__ __forceinline__ bool scatter_stream_switch(ScatterState& c, float* __
 // After the last tile: flushes the accumulate cache (through the bins when there are any; a
 // streaming workgroup has none left) and publishes how many records this workgroup left in each
 // bin.  Call once, by all threads.
-__device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__ level_grad, const BinTarget& bins,
+__device__ __forceinline__ void scatter_end(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group, bool streaming) {
     __syncthreads();
     if (!streaming) cache_flush(c, level_grad, bins, group);
@@ -466,7 +475,7 @@ __device__ __forceinline__ void scatter_end(ScatterState& c, float* __restrict__
 // a plain coalesced read-modify-write; workgroups that share a bin add with atomics (consecutive
 // addresses: one request per 64 bytes).
 __global__ void __launch_bounds__(kReduceBlock)
-bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity,
+bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity, uint32_t feat_pairs,
                   float* __restrict__ table_grad, int first_level) {
     // one array per feature: lanes that hit different slots then spread over all bank pairs (interleaved
     // features would leave every other pair idle in each of the two adds)
@@ -476,7 +485,9 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     // last level first: with the usual coarse-to-fine level list the bins with the most records are
     // started first and the nearly empty ones fill the tail of the launch
     const uint32_t level_in_pass = gridDim.y - 1 - blockIdx.y;
-    const int level = first_level + level_in_pass;
+    // with more than two features per level, every pair of features is scattered and reduced like a level of its own
+    const uint32_t pair_level = static_cast<uint32_t>(first_level) + level_in_pass;
+    const uint32_t level = pair_level / feat_pairs, pair = pair_level % feat_pairs;
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
@@ -537,20 +548,21 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
         }
     }
     __syncthreads();
-    float2* level_grad = reinterpret_cast<float2*>(table_grad + static_cast<size_t>(level) * capacity * 2);
+    const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs};
     const uint32_t slot0 = bin << kBinSlotsLog2;
     const bool alone = gridDim.z == 1;
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
         const double v0 = acc0[s], v1 = acc1[s];
         if ((v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity) {
+            float2* cell = reinterpret_cast<float2*>(level_grad.at(slot0 + s));
             if (alone) {
-                float2 g = level_grad[slot0 + s];
+                float2 g = *cell;
                 g.x += static_cast<float>(v0);
                 g.y += static_cast<float>(v1);
-                level_grad[slot0 + s] = g;
+                *cell = g;
             } else {
-                global_add(&level_grad[slot0 + s].x, static_cast<float>(v0));
-                global_add(&level_grad[slot0 + s].y, static_cast<float>(v1));
+                global_add(&cell->x, static_cast<float>(v0));
+                global_add(&cell->y, static_cast<float>(v1));
             }
         }
     }

@@ -38,9 +38,13 @@ KILLED = [
     ("barycentric index", "s.bary[D - s.rank[i]] += delta;", "s.bary[D1 - s.rank[i]] += delta;"),
     ("barycentric without the wrap-around term", "s.bary[0] += static_cast<R>(1) + s.bary[D1];", "s.bary[0] += static_cast<R>(1);"),
     ("vertex key off by one rank", "if (s.rank[i] > D - r) key[i] -= (D + 1);", "if (s.rank[i] >= D - r) key[i] -= (D + 1);"),
-    ("forward weights reversed", "const R w = s.bary[r] * w_lvl;\n                acc0", "const R w = s.bary[D - r] * w_lvl;\n                acc0"),
-    ("table backward weights reversed", "const R w = s.bary[r] * w_lvl;\n                const R t0", "const R w = s.bary[D - r] * w_lvl;\n                const R t0"),
-    ("table backward swaps the features", "const R t0 = g0 * w, t1 = g1 * w;", "const R t0 = g1 * w, t1 = g0 * w;"),
+    ("forward weights reversed", "const R w = s.bary[r] * w_lvl;\n                for (int f = 0; f < F; ++f) acc[f]",
+     "const R w = s.bary[D - r] * w_lvl;\n                for (int f = 0; f < F; ++f) acc[f]"),
+    ("forward feature stride", "const int64_t h = static_cast<int64_t>(F) * lattice_slot<D>(key, C);\n                const R w = s.bary[r]",
+     "const int64_t h = static_cast<int64_t>(2) * lattice_slot<D>(key, C);\n                const R w = s.bary[r]"),
+    ("table backward weights reversed", "const R w = s.bary[r] * w_lvl;\n                for (int f = 0; f < F; ++f) {\n                    const R t = g[f] * w;",
+     "const R w = s.bary[D - r] * w_lvl;\n                for (int f = 0; f < F; ++f) {\n                    const R t = g[f] * w;"),
+    ("table backward swaps the features", "const R t = g[f] * w;", "const R t = g[F - 1 - f] * w;"),
     ("position backward drops the wrap-around term", "dB[D1] += dB[0];  //", "dB[D1] += 0;  //"),
     ("position backward second index", "dE[i] -= dB[D1 - s.rank[i]] * inv;", "dE[i] -= dB[D - s.rank[i]] * inv;"),
     ("position backward factor", "dP -= dE[i + 1] * sfl[i] * static_cast<R>(i + 1);", "dP -= dE[i + 1] * sfl[i] * static_cast<R>(i);"),
@@ -49,7 +53,9 @@ KILLED = [
     ("double backward factor", "for (int i = 0; i < D; ++i) dE[i + 1] -= q[i] * sf[i] * static_cast<R>(i + 1);",
      "for (int i = 0; i < D; ++i) dE[i + 1] -= q[i] * sf[i] * static_cast<R>(i);"),
     ("double backward prefix sums", "for (int j = 0; j <= i; ++j) dE[j] += g;", "for (int j = 0; j < i; ++j) dE[j] += g;"),
-    ("grad-grad uses the other feature", "gg1 += dB[r] * w_lvl * table[h + 1];", "gg1 += dB[r] * w_lvl * table[h];"),
+    ("grad-grad uses the other feature", "if (ggs) gg[f] += dB[r] * w_lvl * table[h + f];", "if (ggs) gg[f] += dB[r] * w_lvl * table[h + F - 1 - f];"),
+    ("position backward drops a feature", "for (int f = 0; f < F; ++f) {\n                    dB[r] += tl[h + f] * w_lvl * g[f];",
+     "for (int f = 1; f < F; ++f) {\n                    dB[r] += tl[h + f] * w_lvl * g[f];"),
     ("scale factor numerator", "std::sqrt(static_cast<double>((i + 1) * (i + 2)))", "std::sqrt(static_cast<double>((i + 1) * (i + 1)))"),
 ]
 

@@ -22,6 +22,7 @@ from oracle import api as orc
 from helpers import HASH_MUL, random_problem
 
 DIMS = [2, 3, 4, 5, 6, 7, 8]
+FEATS = [2, 4]  # features per level: the reference's value and the first generalisation
 
 
 # ----------------------------------------------------------------------------- hash
@@ -252,17 +253,18 @@ def _collision_free(d, dtype, n=512, levels=4, seed=1, capacity=1 << 22):
     raise AssertionError("no collision-free sample found")
 
 
+@pytest.mark.parametrize("feat", FEATS)
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("d", DIMS)
-def test_forward_reproduces_affine_functions(d, dtype):
+def test_forward_reproduces_affine_functions(d, dtype, feat):
     """Simplex interpolation has linear precision: a table holding a.v + c at every touched vertex v
     must give window * (a.E + c) at the point, whatever the simplex."""
     p, sf, s, cap = _collision_free(d, dtype)
     levels, n = s["slot"].shape[:2]
     rng = np.random.default_rng(7)
-    a = rng.standard_normal((2, d + 1))
-    c = rng.standard_normal(2)
-    table = np.zeros((levels, cap, 2), dtype)
+    a = rng.standard_normal((feat, d + 1))
+    c = rng.standard_normal(feat)
+    table = np.zeros((levels, cap, feat), dtype)
     for l in range(levels):
         k = s["keys"][l].reshape(-1, d + 1).astype(np.float64)
         table[l, s["slot"][l].reshape(-1)] = (k @ a.T + c).astype(dtype)
@@ -273,23 +275,25 @@ def test_forward_reproduces_affine_functions(d, dtype):
     assert np.max(np.abs(out - want)) <= tol * scale
 
 
+@pytest.mark.parametrize("feat", FEATS)
 @pytest.mark.parametrize("d", [2, 3, 4, 8])
-def test_forward_constant_table_and_one_hot(d):
+def test_forward_constant_table_and_one_hot(d, feat):
     p, sf, s, cap = _collision_free(d, np.float32, n=256, levels=3)
     levels, n = s["slot"].shape[:2]
-    table = np.empty((levels, cap, 2), np.float32)
-    table[..., 0] = 2.0
-    table[..., 1] = -3.0
+    table = np.empty((levels, cap, feat), np.float32)
+    consts = np.array([2.0, -3.0, 0.5, 7.0][:feat], np.float32)
+    table[...] = consts
     out = orc.forward(p["pos"], table, sf, p["shift"], p["window"])
-    assert np.allclose(out[:, 0], 2.0 * p["window"][:, None], rtol=1e-5)
-    assert np.allclose(out[:, 1], -3.0 * p["window"][:, None], rtol=1e-5)
-    # one-hot: only vertex r of point 0 at level 1 is set -> output of point 0 is its weight
+    for f in range(feat):
+        assert np.allclose(out[:, f], consts[f] * p["window"][:, None], rtol=1e-5)
+    # one-hot: only feature f of vertex r of point 0 at level 1 is set -> that output of point 0 is the vertex weight
     for r in range(d + 1):
+        f = r % feat
         table[:] = 0
-        table[1, s["slot"][1, 0, r], 0] = 1.0
+        table[1, s["slot"][1, 0, r], f] = 1.0
         out = orc.forward(p["pos"], table, sf, p["shift"], np.ones(levels, np.float32))
-        assert np.isclose(out[1, 0, 0], s["bary"][1, 0, r], rtol=1e-6, atol=1e-7)
-        assert np.all(out[[0, 2]] == 0) and np.all(out[:, 1] == 0)
+        assert np.isclose(out[1, f, 0], s["bary"][1, 0, r], rtol=1e-6, atol=1e-7)
+        assert np.all(out[[0, 2]] == 0) and np.all(np.delete(out, f, axis=1) == 0)
 
 
 def test_forward_window_zero_gives_exact_zero_and_is_linear():
@@ -304,15 +308,16 @@ def test_forward_window_zero_gives_exact_zero_and_is_linear():
     assert np.allclose(out[2], 0.5 * ones[2], rtol=1e-6, atol=1e-7)
 
 
+@pytest.mark.parametrize("feat", FEATS)
 @pytest.mark.parametrize("d", [2, 3, 4, 5])
-def test_forward_concat_points_extra_levels(d):
-    p = random_problem(d, 100, 3, 64, seed=4)
+def test_forward_concat_points_extra_levels(d, feat):
+    p = random_problem(d, 100, 3, 64, seed=4, nr_feat=feat)
     sf = orc.scale_factors(d, p["sigmas"])
     out = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"], concat_points=True, points_scaling=0.25)
-    extra = (d + 1) // 2
-    assert out.shape == (3 + extra, 2, 100)
-    flat = out[3:].reshape(extra * 2, 100)
-    for k in range(extra * 2):
+    extra = -(-d // feat)
+    assert out.shape == (3 + extra, feat, 100)
+    flat = out[3:].reshape(extra * feat, 100)
+    for k in range(extra * feat):
         want = p["pos"][:, k] * np.float32(0.25) if k < d else np.zeros(100, np.float32)
         assert np.array_equal(flat[k], want)
     base = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"])
@@ -321,9 +326,10 @@ def test_forward_concat_points_extra_levels(d):
 
 # ----------------------------------------------------------------------------- gradients
 
+@pytest.mark.parametrize("feat", FEATS)
 @pytest.mark.parametrize("d", DIMS)
-def test_table_backward_is_the_adjoint_of_forward(d):
-    p = random_problem(d, 700, 4, 1 << 9, seed=5, dtype=np.float64)  # small capacity: many collisions
+def test_table_backward_is_the_adjoint_of_forward(d, feat):
+    p = random_problem(d, 700, 4, 1 << 9, seed=5, dtype=np.float64, nr_feat=feat)  # small capacity: many collisions
     sf = orc.scale_factors(d, p["sigmas"]).astype(np.float64)
     out = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"], dtype=np.float64)
     tg = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], 1 << 9, dtype=np.float64)["grad64"]
@@ -342,9 +348,9 @@ def test_table_backward_is_the_adjoint_of_forward(d):
     assert np.all(np.abs(r["grad32"] - r["grad64"]) <= 1e-5 * r["abs64"] + 1e-12)
 
 
-def _interior_points(d, levels, n, seed, margin=0.02):
+def _interior_points(d, levels, n, seed, margin=0.02, feat=2):
     """fp64 problem restricted to points whose barycentric weights are all > margin at every level."""
-    p = random_problem(d, n, levels, 1 << 12, seed=seed, sigma_range=(1.0, 0.1), dtype=np.float64)
+    p = random_problem(d, n, levels, 1 << 12, seed=seed, sigma_range=(1.0, 0.1), dtype=np.float64, nr_feat=feat)
     sf = orc.scale_factors(d, p["sigmas"]).astype(np.float64)
     s = orc.simplex(p["pos"], sf, p["shift"], 1 << 12, dtype=np.float64)
     keep = np.all(s["bary"].min(-1) > margin, axis=0)
@@ -355,10 +361,11 @@ def _interior_points(d, levels, n, seed, margin=0.02):
     return p, sf
 
 
+@pytest.mark.parametrize("feat", FEATS)
 @pytest.mark.parametrize("d", DIMS)
-def test_position_backward_matches_finite_differences(d):
+def test_position_backward_matches_finite_differences(d, feat):
     levels = 3
-    p, sf = _interior_points(d, levels, 4000 if d < 7 else 60000, seed=6, margin=0.02 if d < 6 else 0.005)
+    p, sf = _interior_points(d, levels, 4000 if d < 7 else 60000, seed=6, margin=0.02 if d < 6 else 0.005, feat=feat)
     n = p["pos"].shape[0]
     got = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"], dtype=np.float64)["grad64"]
     h = 1e-6
@@ -378,9 +385,10 @@ def test_position_backward_matches_finite_differences(d):
     assert n > 0
 
 
+@pytest.mark.parametrize("feat", FEATS)
 @pytest.mark.parametrize("d", DIMS)
-def test_double_backward_adjoint_identities(d):
-    p = random_problem(d, 500, 4, 1 << 9, seed=8, dtype=np.float64)
+def test_double_backward_adjoint_identities(d, feat):
+    p = random_problem(d, 500, 4, 1 << 9, seed=8, dtype=np.float64, nr_feat=feat)
     sf = orc.scale_factors(d, p["sigmas"]).astype(np.float64)
     args = (p["pos"], p["table"], sf, p["shift"], p["window"])
     pg = orc.backward_pos(*args, p["grad"], dtype=np.float64)["grad64"]
@@ -400,13 +408,15 @@ def test_double_backward_adjoint_identities(d):
     assert np.all(np.abs(r32["grad32"] - r32["grad64"]) <= 1e-5 * r32["abs64"] + 1e-9)
 
 
-def test_double_backward_concat_levels_are_zero():
+@pytest.mark.parametrize("feat", FEATS)
+def test_double_backward_concat_levels_are_zero(feat):
     d = 3
-    p = random_problem(d, 64, 2, 64, seed=9)
+    p = random_problem(d, 64, 2, 64, seed=9, nr_feat=feat)
     sf = orc.scale_factors(d, p["sigmas"])
-    grad = np.concatenate([p["grad"], np.ones((2, 2, 64), np.float32)])
+    extra = -(-d // feat)
+    grad = np.concatenate([p["grad"], np.ones((extra, feat, 64), np.float32)])
     r = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], grad, concat_points=True)
-    assert r["ggs"].shape == (4, 2, 64) and np.all(r["ggs"][2:] == 0)
+    assert r["ggs"].shape == (2 + extra, feat, 64) and np.all(r["ggs"][2:] == 0)
     r0 = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"])
     assert np.array_equal(r["ggs"][:2], r0["ggs"]) and np.array_equal(r["grad64"], r0["grad64"])
 
