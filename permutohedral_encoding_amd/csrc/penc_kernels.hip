@@ -153,7 +153,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
                       const float* __restrict__ grad_sliced, int64_t grad_row_stride,
                       const float* __restrict__ double_pos_grad, float* __restrict__ table_grad,
                       float* __restrict__ grad_level_major, BinTarget pass_bins) {
-    __shared__ ScatterState state;
+    __shared__ ScatterStateT<stage_chunk(D)> state;
     // Workgroups are dealt round-robin to the kXcds dies, each with an L2 of its own.  The j-th
     // workgroup of a die takes level j % levels of one group of points: a die works through all
     // levels of a group before the next group, so the points are fetched from memory once, and
@@ -255,7 +255,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
 // ------------------------------------------------------------------------------------------
 // backward w.r.t. positions (EncodingGPU.cuh:530-769)
 
-// One thread per (point, group of consecutive levels): the levels of the group are summed in
+// One thread per (point, group of levels): the levels of the group are summed in
 // registers and stored once, at out[group][point][D].  With a single group (no workspace) `out` is
 // the position gradient itself; otherwise it is a partial buffer that reduce_level_groups_kernel
 // sums, in ascending group order, so the result is deterministic either way.  Small groups keep
@@ -273,9 +273,13 @@ backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t c
     if (n >= n_points) return;
     const fvec<D> pos = load_point<D>(positions, n);
     fvec<D> total = 0.0f;
-    const int first = blockIdx.y * levels_per_group;
-    const int last = first + levels_per_group < n_levels ? first + levels_per_group : n_levels;
-    for (int level = first; level < last; ++level) {
+    // The levels of a group are `gridDim.y` apart, not adjacent: with the usual coarse-to-fine level list a
+    // group then pairs a coarse level, whose points share few slots, with a fine one, and the table slices
+    // the whole chip gathers from at any time fit the L2 (two adjacent fine levels are 4 MiB at 2^18 slots,
+    // an L2's whole capacity).
+    for (int k = 0; k < levels_per_group; ++k) {
+        const int level = static_cast<int>(blockIdx.y) + k * static_cast<int>(gridDim.y);
+        if (level >= n_levels) break;
         const float w_level = window[level];
         if (w_level == 0.0f) continue;
         const float* sf = scale_factor + level * D;

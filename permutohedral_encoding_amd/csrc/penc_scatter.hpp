@@ -38,15 +38,22 @@ namespace penc {
 
 constexpr int kXcds = 8;               // accelerator dies (XCDs) of the chip; workgroup i runs on die i % kXcds
 constexpr int kBlock = 256;            // threads per workgroup of the gather-type kernels (4 wavefronts)
-constexpr int kScatterBlock = 512;     // threads per scattering workgroup (8 wavefronts share one accumulate cache)
-constexpr int kScatterTiles = 8;       // tiles of kScatterBlock points a scattering workgroup walks (a "group" of points) ...
-constexpr int kScatterTilesLarge = 16; // ... or this many, when the launch still has workgroups to spare
-constexpr int kCacheLinesLog2 = 11;
+#ifndef PENC_SCATTER_BLOCK
+#define PENC_SCATTER_BLOCK 512
+#define PENC_SCATTER_TILES 8
+#define PENC_SCATTER_TILES_LARGE 16
+#define PENC_CACHE_LINES_LOG2 11
+#endif
+constexpr int kScatterBlock = PENC_SCATTER_BLOCK;  // threads per scattering workgroup (its wavefronts share one accumulate cache)
+constexpr int kScatterTiles = PENC_SCATTER_TILES;  // tiles of kScatterBlock points a scattering workgroup walks (a "group" of points) ...
+constexpr int kScatterTilesLarge = PENC_SCATTER_TILES_LARGE;  // ... or this many, when the launch still has workgroups to spare
+constexpr int kCacheLinesLog2 = PENC_CACHE_LINES_LOG2;
 constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per workgroup
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
 constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space
-constexpr int kStageChunk = 5;         // vertices per thread a wave sorts by bin in one go (320 records)
+// vertices per thread a wave sorts by bin in one go (256 or 320 records): all D+1 of them up to D = 4
+constexpr int stage_chunk(int pos_dim) { return pos_dim + 1 <= 4 ? 4 : 5; }
 constexpr int kStageBins = 64;         // a wave counts one bin per lane: staging needs n_bins <= 64
 constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
@@ -170,16 +177,21 @@ __device__ __forceinline__ void global_add_pairs(const GradSlice& level_grad, bo
 // lines are hit by many lanes at once (that is what the cache is for), where a compare-and-swap
 // loop degrades quadratically (measured: 10-40x slower on the coarsest levels) and ds_add_f32 is
 // slow on this chip.  The fp64 partial sums are rounded to fp32 once, when the cache is flushed.
-struct ScatterState {
+template <int kStageChunk>
+struct ScatterStateT {
+    static constexpr int kChunk = kStageChunk;
+    static constexpr int kTail = (kScatterBlock / 64) * kStageChunk * 64 - kCacheLines;
+    static_assert(kTail >= 0, "the staging slices cover the cache's values");
     int tag[kCacheLines];
     double val[2][kCacheLines];  // one array per feature: random lines then spread over all LDS bank pairs
     // when the workgroup streams, val and this tail together are its waves' staging slices
-    uint4 stage_tail[(kScatterBlock / 64) * kStageChunk * 64 - kCacheLines];
+    uint4 stage_tail[kTail > 0 ? kTail : 1];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
     uint32_t hits;                 // contributions the cache has absorbed into existing lines
 };
 
-__device__ __forceinline__ void scatter_begin(ScatterState& c) {
+template <typename State>
+__device__ __forceinline__ void scatter_begin(State& c) {
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         c.tag[e] = -1;
         c.val[0][e] = 0.0;
@@ -192,7 +204,8 @@ __device__ __forceinline__ void scatter_begin(ScatterState& c) {
 
 // Stage 2 for one contribution: append a record to this workgroup's segment of the slot's bin.
 // Returns false when the segment is full.
-__device__ __forceinline__ bool append_record(ScatterState& c, const BinTarget& bins, uint32_t group, uint32_t slot,
+template <typename State>
+__device__ __forceinline__ bool append_record(State& c, const BinTarget& bins, uint32_t group, uint32_t slot,
                                               float a0, float a1) {
     const uint32_t b = slot >> kBinSlotsLog2;
     const uint32_t pos = atomicAdd(&c.bin_count[b], 1u);
@@ -212,7 +225,8 @@ __device__ __forceinline__ bool append_record(ScatterState& c, const BinTarget& 
 // line already held the slot (a hit, as opposed to a claim).
 // (Spreading the lanes that share a slot over replicated sub-tables, instead of folding them in
 // registers first, was measured 30% slower on the coarse levels, and no faster on top of folding.)
-__device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& found) {
+template <typename State>
+__device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) {
     const int want = static_cast<int>(slot);
     int e = static_cast<int>(slot & (kCacheLines - 1));
     found = false;
@@ -233,7 +247,7 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
 }
 
 // Stage 2 for a whole tile once the workgroup streams (see scatter_stream_switch): the cache's LDS
-// is staging space, a 5 KiB slice per wave.  For kStageChunk vertices per thread at a time, the wave
+// is staging space, a 4 or 5 KiB slice per wave.  For stage_chunk(D) vertices per thread at a time, the wave
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
 // its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
@@ -243,14 +257,15 @@ __device__ __forceinline__ int cache_find(ScatterState& c, uint32_t slot, bool& 
 // every record against the room left and sends the excess to stage 3.
 // Needs bins.n_bins <= kStageBins and a level's record array below 2^32 bytes (the host plans
 // for both); all 64 lanes of the wave must call it together.
-template <int D>
-__device__ __forceinline__ void stream_tile(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
+template <int D, typename State>
+__device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
                                             fvec<D + 1> a1) {
     constexpr int kWaves = kScatterBlock / 64;
+    constexpr int kStageChunk = State::kChunk;
     static_assert(kCacheLines / kWaves >= 4 * 64, "four 64-entry arrays per wave live in the tag array");
-    static_assert(offsetof(ScatterState, stage_tail) == offsetof(ScatterState, val) + sizeof(c.val) &&
-                      (sizeof(c.val) + sizeof(c.stage_tail)) / kWaves == kStageChunk * 64 * sizeof(uint4),
+    static_assert(offsetof(State, stage_tail) == offsetof(State, val) + sizeof(c.val) &&
+                      (sizeof(c.val) + (State::kTail > 0 ? sizeof(c.stage_tail) : 0)) / kWaves == kStageChunk * 64 * sizeof(uint4),
                   "val and stage_tail are one contiguous array of staging slices");
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     uint32_t* count = reinterpret_cast<uint32_t*>(c.tag) + wave * (kCacheLines / kWaves);  // records per bin
@@ -356,8 +371,8 @@ __device__ __forceinline__ void stream_tile(ScatterState& c, const GradSlice& le
 // only take part in the wave-wide steps.  `use_cache` (wave-uniform) is false once the workgroup
 // has seen that the cache does not hit at this level; `streaming` is what scatter_stream_switch
 // returned.  The return value is the number of hits of this wave in this tile.
-template <int D>
-__device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
+template <int D, typename State>
+__device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
                                                  uint32_t group, bool active, bool use_cache, bool streaming,
                                                  uvec<D + 1> slot, fvec<D + 1> a0, fvec<D + 1> a1) {
     if (streaming) {
@@ -412,13 +427,14 @@ __device__ __forceinline__ uint32_t scatter_tile(ScatterState& c, const GradSlic
 
 // The workgroup-wide decision whether stage 1 is worth its LDS traffic at this level: after the
 // first tile, keep using the cache only while at least one contribution in eight hits.
-template <int D>
-__device__ __forceinline__ bool cache_pays(const ScatterState& c, int tiles_done) {
+template <int D, typename State>
+__device__ __forceinline__ bool cache_pays(const State& c, int tiles_done) {
     return tiles_done == 0 || c.hits * 8u >= static_cast<uint32_t>(tiles_done) * kScatterBlock * (D + 1);
 }
 
 // Sends every line of the accumulate cache on to stage 2 (or 3).  By all threads, between barriers.
-__device__ __forceinline__ void cache_flush(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
+template <typename State>
+__device__ __forceinline__ void cache_flush(State& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group) {
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
         const int owner = c.tag[e];
@@ -437,8 +453,8 @@ __device__ __forceinline__ void cache_flush(ScatterState& c, const GradSlice& le
 // Before tile `tile` (all threads call it, with the same arguments): decides for the whole
 // workgroup whether to give up the accumulate cache for good and use its LDS as staging space
 // (stream_tile).  Returns true from then on; the cache's contents have been flushed by then.
-template <int D>
-__device__ __forceinline__ bool scatter_stream_switch(ScatterState& c, const GradSlice& level_grad,
+template <int D, typename State>
+__device__ __forceinline__ bool scatter_stream_switch(State& c, const GradSlice& level_grad,
                                                       const BinTarget& bins, uint32_t group, int tile) {
     if (tile != kStreamDecisionTile || bins.records == nullptr || bins.n_bins > kStageBins) return false;
     __syncthreads();  // the hits of the tiles so far are in
@@ -453,7 +469,8 @@ __device__ __forceinline__ bool scatter_stream_switch(ScatterState& c, const Gra
 // After the last tile: flushes the accumulate cache (through the bins when there are any; a
 // streaming workgroup has none left) and publishes how many records this workgroup left in each
 // bin.  Call once, by all threads.
-__device__ __forceinline__ void scatter_end(ScatterState& c, const GradSlice& level_grad, const BinTarget& bins,
+template <typename State>
+__device__ __forceinline__ void scatter_end(State& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group, bool streaming) {
     __syncthreads();
     if (!streaming) cache_flush(c, level_grad, bins, group);
