@@ -11,9 +11,9 @@
  *  - Plain pointers and sizes only.  Unless a parameter says "host", every pointer is DEVICE
  *    memory of the GPU that is current on the calling thread; it is borrowed for the duration of
  *    the enqueued work.  The library never allocates or frees device memory and keeps no state.
- *  - All arrays are fp32, densely packed, row-major (F = nr_feat, the features per level):
+ *  - All arrays are fp32, densely packed, row-major (F = nr_feat, the features per level: 2, 4 or 8):
  *        positions            [N][D]
- *        lattice_values       [L][C][F]      (aligned to one slot: 8 bytes for F = 2, 16 for F = 4)
+ *        lattice_values       [L][C][F]      (8-byte aligned for F = 2, 16-byte for F = 4 and 8)
  *        scale_factor         [L][D]         (from penc_scale_factors)
  *        random_shift         [L][D]
  *        anneal_window        [L]
@@ -30,9 +30,10 @@
  *    depend on it beyond the order of floating-point accumulation.
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Work is enqueued and
  *    the call returns without synchronising, like the reference's launches on the current stream.
- *  - D = pos_dim in 2..8, nr_feat 2 or 4 (reference: Encoding.cuh:139-156 supports 2..7 and 2 only; its
- *    instantiations for 4 and 8 features are commented out, src/Encoding.cu:362-363).  With four
- *    features the table gradient treats the feature pairs (0,1) and (2,3) of a level like two levels.
+ *  - D = pos_dim in 2..8, nr_feat 2, 4 or 8 (reference: Encoding.cuh:139-156 supports 2..7 and 2 only;
+ *    its instantiations for 4 and 8 features are commented out, src/Encoding.cu:362-363).  With more
+ *    than two features the table gradient treats the feature pairs (0,1), (2,3), ... of a level like
+ *    levels of their own.
  *  - Every function returns PENC_OK or one of the error codes below; penc_status_string() names it.
  */
 #ifndef PENC_H_
@@ -49,7 +50,7 @@ extern "C" {
 #define PENC_ERR_NULL_POINTER 1        /* a required pointer is NULL */
 #define PENC_ERR_BAD_SIZE 2            /* N, L or C is not positive, or a product overflows 2^31 elements */
 #define PENC_ERR_UNSUPPORTED_POS_DIM 3 /* pos_dim outside 2..8 (reference: Encoding.cuh:155) */
-#define PENC_ERR_UNSUPPORTED_NR_FEAT 4 /* nr_feat not 2 or 4 (reference: Encoding.cuh:142 accepts 2 only) */
+#define PENC_ERR_UNSUPPORTED_NR_FEAT 4 /* nr_feat not 2, 4 or 8 (reference: Encoding.cuh:142 accepts 2 only) */
 #define PENC_ERR_MISALIGNED 5          /* lattice_values not aligned to a slot, or a gradient array not to 8 bytes */
 #define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
 #define PENC_ERR_SCRATCH_TOO_SMALL 7    /* penc_backward_static: the problem does not fit the static scratch */

@@ -175,7 +175,7 @@ def is_row_major_view(grad):
         return False
     levels, feat, n = grad.shape
     s_level, s_feat, s_point = grad.stride()
-    return (feat in (2, 4) and n > 0 and s_level == feat and s_feat == 1 and s_point >= feat * levels and s_point % 2 == 0
+    return (feat in (2, 4, 8) and n > 0 and s_level == feat and s_feat == 1 and s_point >= feat * levels and s_point % 2 == 0
             and grad.data_ptr() % 8 == 0 and s_point * n < 2 ** 31)
 
 
@@ -234,8 +234,8 @@ class EncodingWrapper:
     """The native encoding object (reference: ``EncodingWrapper``, Encoding.cuh:162-188)."""
 
     def __init__(self, pos_dim, nr_feat_per_level, fixed_params):
-        if nr_feat_per_level not in (2, 4):
-            raise RuntimeError("Encoding: nr_feat_per_level must be 2 or 4")
+        if nr_feat_per_level not in (2, 4, 8):
+            raise RuntimeError("Encoding: nr_feat_per_level must be 2, 4 or 8")
         if pos_dim not in (2, 3, 4, 5, 6, 7, 8):
             raise RuntimeError("Encoding: pos_dim must be 2,3,4,5,6,7 or 8")
         self.pos_dim = int(pos_dim)

@@ -41,7 +41,7 @@ __device__ __forceinline__ fvec<D> load_point(const float* __restrict__ position
     return pos;
 }
 
-// The D+1 table entries of a simplex (F features each: one 8- or 16-byte load per vertex), fetched
+// The D+1 table entries of a simplex (F features each: an 8-byte or one or two 16-byte loads per vertex), fetched
 // back to back so that all loads are in flight together.  f[k][r] is feature k of vertex r.
 template <int D, int F>
 struct Vertices {
@@ -50,7 +50,7 @@ struct Vertices {
 template <int D, int F>
 __device__ __forceinline__ Vertices<D, F> load_vertices(const float* __restrict__ level_table, uvec<D + 1> h,
                                                         uint32_t capacity, uint32_t cap_mask) {
-    static_assert(F == 2 || F == 4, "two or four features per level");
+    static_assert(F == 2 || F == 4 || F == 8, "two, four or eight features per level");
     Vertices<D, F> v;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
@@ -60,11 +60,14 @@ __device__ __forceinline__ Vertices<D, F> load_vertices(const float* __restrict_
             v.f[0][r] = x.x;
             v.f[1][r] = x.y;
         } else {
-            const float4 x = *reinterpret_cast<const float4*>(level_table + 4 * slot);
-            v.f[0][r] = x.x;
-            v.f[1][r] = x.y;
-            v.f[2][r] = x.z;
-            v.f[3][r] = x.w;
+            static_for<F / 4>(PENC_BODY(q) {
+                PENC_INDEX(q);
+                const float4 x = *reinterpret_cast<const float4*>(level_table + F * slot + 4 * q);
+                v.f[4 * q + 0][r] = x.x;
+                v.f[4 * q + 1][r] = x.y;
+                v.f[4 * q + 2][r] = x.z;
+                v.f[4 * q + 3][r] = x.w;
+            });
         }
     });
     return v;
@@ -140,7 +143,7 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 // kSecondOrder: the table-gradient half of the double backward (EncodingGPU.cuh:1016-1257): the
 // vertex weights are the derivatives of the barycentric weights along `double_pos_grad` instead of
 // the barycentric weights themselves; everything else is the same scatter.
-// feat_pairs: with four features per level the pairs (0,1) and (2,3) are scattered like two levels that
+// feat_pairs: with four or eight features per level the pairs (0,1), (2,3), ... are scattered like levels that
 // share their geometry: "levels" below (first_level, n_pass_levels, the grid, the bins) count pairs,
 // `pair_level` = level * feat_pairs + pair.  The upstream gradient needs no special case: [L][F][N]
 // is [L * F/2][2][N], and in a row the pair sits at column 2 * pair_level.
@@ -454,7 +457,7 @@ inline uint32_t mask_of(int capacity) {
 
 inline int check_geometry(int pos_dim, int nr_feat, int64_t n, int levels, int capacity, int extra) {
     if (pos_dim < 2 || pos_dim > 8) return PENC_ERR_UNSUPPORTED_POS_DIM;
-    if (nr_feat != 2 && nr_feat != 4) return PENC_ERR_UNSUPPORTED_NR_FEAT;
+    if (nr_feat != 2 && nr_feat != 4 && nr_feat != 8) return PENC_ERR_UNSUPPORTED_NR_FEAT;
     if (n <= 0 || levels <= 0 || capacity <= 0) return PENC_ERR_BAD_SIZE;
     const int64_t lim = (int64_t{1} << 31) - 1;
     if (n > lim / (nr_feat * (int64_t{levels} + extra)) || n > lim / pos_dim) return PENC_ERR_BAD_SIZE;
@@ -464,8 +467,8 @@ inline int check_geometry(int pos_dim, int nr_feat, int64_t n, int levels, int c
 }
 
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
-// the table is gathered with one load per slot: 8 bytes for two features, 16 for four
-inline bool table_aligned(const void* p, int nr_feat) { return (reinterpret_cast<uintptr_t>(p) & (nr_feat == 4 ? 15u : 7u)) == 0; }
+// the table is gathered with 8-byte loads for two features and 16-byte loads for four or eight
+inline bool table_aligned(const void* p, int nr_feat) { return (reinterpret_cast<uintptr_t>(p) & (nr_feat >= 4 ? 15u : 7u)) == 0; }
 
 // Clears the table gradient with a fill kernel (float2 granularity: the array is only guaranteed
 // 8-byte alignment).  A kernel rather than hipMemsetAsync so that callers may capture the call in
@@ -588,9 +591,12 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
         default: return PENC_ERR_UNSUPPORTED_POS_DIM;              \
     }
 
-// The same with the number of features per level (2 or 4) as the constant FF.
+// The same with the number of features per level (2, 4 or 8) as the constant FF.
 #define PENC_DISPATCH_DF(D_, F_, ...)                                   \
-    if ((F_) == 4) {                                                    \
+    if ((F_) == 8) {                                                    \
+        constexpr int FF = 8;                                           \
+        PENC_DISPATCH_D(D_, __VA_ARGS__)                                \
+    } else if ((F_) == 4) {                                             \
         constexpr int FF = 4;                                           \
         PENC_DISPATCH_D(D_, __VA_ARGS__)                                \
     } else {                                                            \
@@ -745,8 +751,8 @@ const char* penc_status_string(int status) {
         case PENC_ERR_NULL_POINTER: return "a required pointer is NULL";
         case PENC_ERR_BAD_SIZE: return "nr_positions, nr_levels and capacity must be positive and every array must stay below 2^31 elements";
         case PENC_ERR_UNSUPPORTED_POS_DIM: return "pos_dim must be 2,3,4,5,6,7 or 8";
-        case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2 or 4";
-        case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to one slot (8 bytes for two features, 16 for four), lattice_values_grad and gradient rows to 8 bytes";
+        case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2, 4 or 8";
+        case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to 8 bytes for two features per level and to 16 for four or eight, lattice_values_grad and gradient rows to 8 bytes";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
         case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major copy of the upstream gradient (penc_backward_rowmajor_workspace_bytes)";
         case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
@@ -856,7 +862,7 @@ static int check_rows(const float* grad_rows, int64_t grad_row_stride, int64_t n
 
 size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
                                               int want_lattice_values_grad, int want_positions_grad) {
-    if (pos_dim < 2 || pos_dim > 8 || (nr_feat != 2 && nr_feat != 4) || nr_positions <= 0 || nr_levels <= 0 || capacity <= 0)
+    if (pos_dim < 2 || pos_dim > 8 || (nr_feat != 2 && nr_feat != 4 && nr_feat != 8) || nr_positions <= 0 || nr_levels <= 0 || capacity <= 0)
         return 0;
     size_t scratch = 0;
     if (want_lattice_values_grad)

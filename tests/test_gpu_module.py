@@ -337,25 +337,26 @@ def test_row_major_backward_needs_room_for_the_copy():
     assert rc == 8 and b"level-major copy" in lib.penc_status_string(rc)
 
 
-def test_module_with_four_features_per_level():
-    """PermutoEncoding(..., nr_feat_per_level=4): output layout (column = level * 4 + feature), training
-    step and eikonal-style double backward through autograd, against the oracle."""
+@pytest.mark.parametrize("feat", [4, 8])
+def test_module_with_more_features_per_level(feat):
+    """PermutoEncoding(..., nr_feat_per_level=4 or 8): output layout (column = level * F + feature),
+    training step and eikonal-style double backward through autograd, against the oracle."""
     import permutohedral_encoding_amd as pe
     torch.manual_seed(1)
     levels, n = 5, 3000
-    m = pe.PermutoEncoding(3, 1 << 12, levels, 4, np.geomspace(1.0, 1e-2, levels))
+    m = pe.PermutoEncoding(3, 1 << 12, levels, feat, np.geomspace(1.0, 1e-2, levels))
     with torch.no_grad():
         m.lattice_values.uniform_(-1, 1)
     pos = torch.rand(n, 3, device="cuda", requires_grad=True)
     out = m(pos)
-    assert out.shape == (n, 20) == (n, m.output_dims())
+    assert out.shape == (n, levels * feat) == (n, m.output_dims())
     p, t, sf, sh = oracle_args(m, pos)
     w = np.ones(levels, np.float32)
     want = orc.forward(p, t, sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
     assert np.array_equal(out.detach().cpu().numpy(), want)
-    up = torch.randn(n, 20, device="cuda")
+    up = torch.randn(n, levels * feat, device="cuda")
     grad_pos, = torch.autograd.grad(out, pos, up, create_graph=True)
-    g = up.cpu().numpy().reshape(n, levels, 4).transpose(1, 2, 0).copy()
+    g = up.cpu().numpy().reshape(n, levels, feat).transpose(1, 2, 0).copy()
     wp = orc.backward_pos(p, t, sf, sh, w, g)
     assert np.all(np.abs(grad_pos.detach().cpu().numpy() - wp["grad64"]) <= 1e-6 * wp["abs64"] + 1e-30)
     q = torch.randn(n, 3, device="cuda")

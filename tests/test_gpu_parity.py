@@ -174,54 +174,56 @@ def test_all_dims_all_phases_match_oracle(d):
     check_grad_grad(ggs.cpu().numpy(), want)
 
 
-# ----------------------------------------------------------------------------- four features per level
+# ----------------------------------------------------------------------------- four and eight features per level
 
+@pytest.mark.parametrize("feat", [4, 8])
 @pytest.mark.parametrize("d", DIMS)
-def test_four_features_per_level_all_phases_match_oracle(d):
-    """nr_feat_per_level = 4 (the reference stops at 2): same algorithm, 16-byte slots; the table gradient
-    scatters the feature pairs (0,1) and (2,3) like two levels.  All phases against the oracle."""
+def test_more_features_per_level_all_phases_match_oracle(d, feat):
+    """nr_feat_per_level = 4 and 8 (the reference stops at 2): same algorithm, 16- and 32-byte slots; the
+    table gradient scatters the feature pairs (0,1), (2,3), ... like levels.  All phases against the oracle."""
     cap = (1 << 12) if d != 4 else 5000  # one capacity that is not a power of two
     n, levels = 6000, 5
-    p = random_problem(d, n, levels, cap, seed=60 + d, sigma_range=(1.0, 1e-3), nr_feat=4)
+    p = random_problem(d, n, levels, cap, seed=60 + d + feat, sigma_range=(1.0, 1e-3), nr_feat=feat)
     sf = orc.scale_factors(d, p["sigmas"])
-    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=4)
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
     inp = gpu_input(p)
     out = enc.forward(inp).cpu().numpy()
     want = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"])
-    assert out.shape == (levels, 4, n)
+    assert out.shape == (levels, feat, n)
     check_forward(out, want)
     assert np.array_equal(out, want)
     tg, pg = enc.backward(inp, to_gpu(p["grad"]))
     want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
-    assert tg.shape == (levels, cap, 4)
-    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient, four features")
+    assert tg.shape == (levels, cap, feat)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient, %d features" % feat)
     check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"]))
     tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
     want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
-    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient, four features")
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "double-backward table gradient, %d features" % feat)
     check_grad_grad(ggs.cpu().numpy(), want)
 
 
-def test_four_features_at_benchmark_size_with_rows_and_concat_points():
-    """The headline geometry (3-D, 24 levels, 2^18 slots) with four features per level at 2^18 points:
-    binned scatter over 48 feature pairs, the upstream gradient given as rows of 4 * (24 + 1) columns."""
+@pytest.mark.parametrize("feat,n", [(4, 1 << 18), (8, 1 << 17)])
+def test_more_features_at_benchmark_size_with_rows_and_concat_points(feat, n):
+    """The headline geometry (3-D, 24 levels, 2^18 slots) with four and eight features per level: binned
+    scatter over 48 and 96 feature pairs, the upstream gradient given as rows of F * (24 + 1) columns."""
     from permutohedral_encoding_amd import _native
-    d, n, levels, cap = 3, 1 << 18, 24, 1 << 18
-    p = random_problem(d, n, levels, cap, seed=71, sigma_range=(1.0, 1e-4), nr_feat=4)
+    d, levels, cap = 3, 24, 1 << 18
+    p = random_problem(d, n, levels, cap, seed=71, sigma_range=(1.0, 1e-4), nr_feat=feat)
     p["table"] *= 1e-2
     sf = orc.scale_factors(d, p["sigmas"])
-    enc, _ = make_encoding(d, p["sigmas"], p["shift"], concat_points=True, points_scaling=0.5, nr_feat=4)
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], concat_points=True, points_scaling=0.5, nr_feat=feat)
     inp = gpu_input(p)
     out = enc.forward(inp).cpu().numpy()
     want = orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"], concat_points=True, points_scaling=0.5)
-    assert out.shape == (levels + 1, 4, n) and np.array_equal(out, want)
-    rows = torch.randn(n, 4 * (levels + 1), device="cuda")
-    view = rows.reshape(n, levels + 1, 4).permute(1, 2, 0)
+    assert out.shape == (levels + 1, feat, n) and np.array_equal(out, want)
+    rows = torch.randn(n, feat * (levels + 1), device="cuda")
+    view = rows.reshape(n, levels + 1, feat).permute(1, 2, 0)
     assert _native.is_row_major_view(view)
     level_major = np.ascontiguousarray(view[:levels].cpu().numpy())
     tg, pg = enc.backward(inp, view)
     want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], level_major, cap, want32=False, want_abs=True)
-    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient from rows, four features")
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient from rows, %d features" % feat)
     check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], level_major))
     tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), view)
     want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], level_major,
@@ -333,7 +335,7 @@ def test_error_paths():
     with pytest.raises(RuntimeError, match="pos_dim"):
         _native.EncodingWrapper.create(9, 2, None)
     with pytest.raises(RuntimeError, match="nr_feat_per_level"):
-        _native.EncodingWrapper.create(3, 8, None)
+        _native.EncodingWrapper.create(3, 16, None)
     # strided positions are accepted (the reference indexes through accessors)
     pos2 = to_gpu(np.concatenate([p["pos"], p["pos"]], axis=1))[:, :3]
     out = enc.forward(_native.EncodingInput(good.m_lattice_values, pos2, good.m_anneal_window, True, True))

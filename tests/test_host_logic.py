@@ -42,7 +42,7 @@ def test_status_strings_and_extra_levels():
     lib = _native.lib()
     assert lib.penc_status_string(0) == b"ok"
     assert b"pos_dim" in lib.penc_status_string(3)
-    assert b"nr_feat_per_level must be 2 or 4" in lib.penc_status_string(4)
+    assert b"nr_feat_per_level must be 2, 4 or 8" in lib.penc_status_string(4)
     for d in range(2, 9):
         assert _native.extra_levels(d, 2, False) == 0
         assert _native.extra_levels(d, 2, True) == math.ceil(d / 2) == orc.extra_levels(d, True)
@@ -56,7 +56,7 @@ def test_argument_validation_without_a_gpu():
     p = buf.ctypes.data
     assert lib.penc_forward(9, 2, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 3
     assert lib.penc_forward(1, 2, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 3
-    assert lib.penc_forward(3, 8, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 4
+    assert lib.penc_forward(3, 16, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 4
     assert lib.penc_forward(3, 3, 10, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 4
     assert lib.penc_forward(3, 4, 10, 2, 16, p, p + 8, p, p, p, p, 0, 1.0, None) == 5  # four features: 16-byte slots
     assert lib.penc_forward(3, 2, 0, 2, 16, p, p, p, p, p, p, 0, 1.0, None) == 2
@@ -136,7 +136,7 @@ def test_module_surface_on_cpu():
     with pytest.raises(ValueError, match="GPU memory"):
         m(torch.rand(4, 3))
     with pytest.raises(RuntimeError, match="nr_feat_per_level"):
-        pe.PermutoEncoding(3, 64, 2, 8, [1.0, 0.5], device="cpu")
+        pe.PermutoEncoding(3, 64, 2, 6, [1.0, 0.5], device="cpu")
     m4 = pe.PermutoEncoding(3, 64, 2, 4, [1.0, 0.5], concat_points=True, device="cpu")   # four features per level
     assert m4.lattice_values.shape == (2, 64, 4) and m4.output_dims() == 4 * (2 + 1)
     with pytest.raises(RuntimeError, match="pos_dim"):

@@ -22,7 +22,7 @@ from oracle import api as orc
 from helpers import HASH_MUL, random_problem
 
 DIMS = [2, 3, 4, 5, 6, 7, 8]
-FEATS = [2, 4]  # features per level: the reference's value and the first generalisation
+FEATS = [2, 4, 8]  # features per level: the reference's value and the two generalisations its text anticipates
 
 
 # ----------------------------------------------------------------------------- hash
@@ -281,7 +281,7 @@ def test_forward_constant_table_and_one_hot(d, feat):
     p, sf, s, cap = _collision_free(d, np.float32, n=256, levels=3)
     levels, n = s["slot"].shape[:2]
     table = np.empty((levels, cap, feat), np.float32)
-    consts = np.array([2.0, -3.0, 0.5, 7.0][:feat], np.float32)
+    consts = np.array([2.0, -3.0, 0.5, 7.0, -1.5, 4.0, 0.25, -8.0][:feat], np.float32)
     table[...] = consts
     out = orc.forward(p["pos"], table, sf, p["shift"], p["window"])
     for f in range(feat):
