@@ -525,10 +525,45 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     // chunks of kUnroll wave-widths, and the next chunk's loads are issued before the current
     // chunk's LDS atomics, so a wave always has loads in flight.
     constexpr uint32_t kChunk = 64 * kUnroll;
+    // Short segments (a large table has hundreds of bins, so a scattering workgroup leaves only a few
+    // dozen records in each): a quarter of the wave per segment, four segments at a time, each taken
+    // whole in one step of kShortUnroll loads per lane.
+    constexpr uint32_t kShortLanes = 16, kShortUnroll = 8, kShortMax = kShortLanes * kShortUnroll;
     for (uint32_t g0 = group_begin + wave; g0 < group_end; g0 += kWaves * 64) {
         const uint32_t mine = g0 + lane * kWaves;
         const uint32_t my_count = mine < group_end ? counts[mine] : 0u;
         const uint32_t n_segments = (group_end - g0 + kWaves - 1) / kWaves < 64u ? (group_end - g0 + kWaves - 1) / kWaves : 64u;
+        if (__ballot(my_count > kShortMax) == 0ull) {
+            const uint32_t quarter = lane / kShortLanes, l = lane % kShortLanes;
+            const uint32_t n_steps = (n_segments + 3) / 4;
+            const auto fetch4 = [&](uint32_t step, BinRecord (&rec)[kShortUnroll]) {
+                const uint32_t k = 4 * step + quarter;  // < 64; lanes past the last segment hold a count of 0
+                const uint32_t count = static_cast<uint32_t>(__shfl(static_cast<int>(my_count), static_cast<int>(k)));
+                const BinRecord* seg = recs + static_cast<size_t>(g0 + k * kWaves) * bins.segment_capacity;
+#pragma unroll
+                for (uint32_t u = 0; u < kShortUnroll; ++u) {
+                    const uint32_t i = u * kShortLanes + l;
+                    rec[u] = *(i < count ? seg + i : recs);  // the bin's first record stands in where there is none
+                }
+                return count;
+            };
+            BinRecord cur[kShortUnroll], next[kShortUnroll];
+            uint32_t cur_count = fetch4(0, cur), next_count = 0;
+            for (uint32_t step = 0; step < n_steps; ++step) {
+                if (step + 1 < n_steps) next_count = fetch4(step + 1, next);
+#pragma unroll
+                for (uint32_t u = 0; u < kShortUnroll; ++u)
+                    if (u * kShortLanes + l < cur_count) {
+                        const uint32_t cell = cur[u].slot_in_bin;
+                        __hip_atomic_fetch_add(&acc0[cell], static_cast<double>(cur[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                        __hip_atomic_fetch_add(&acc1[cell], static_cast<double>(cur[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    }
+#pragma unroll
+                for (uint32_t u = 0; u < kShortUnroll; ++u) cur[u] = next[u];
+                cur_count = next_count;
+            }
+            continue;
+        }
         const auto count_of = [&](uint32_t k) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(my_count, k)); };
         const auto fetch = [&](uint32_t k, uint32_t base, BinRecord (&rec)[kUnroll]) {
             const uint32_t count = count_of(k);
