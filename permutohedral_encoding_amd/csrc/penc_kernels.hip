@@ -212,7 +212,8 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     if constexpr (kSecondOrder) q = load_group_point(group_q, nn);
     float g0, g1;
     load_grad(nn, g0, g1);
-    bool streaming = false;
+    int mode = kModeCache;
+    uint32_t id_bits = 0;
     for (int t = 0; t < tiles_per_group; ++t) {
         const int64_t tile_base = group_base + static_cast<int64_t>(t) * kScatterBlock;
         if (tile_base >= n_points) break;
@@ -230,7 +231,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
                 out[n_points] = g1;
             }
         }
-        if (!streaming) streaming = scatter_stream_switch<D>(state, level_grad, bins, group, t);
+        if (t == kStreamDecisionTile) mode = scatter_mode_switch<D>(state, level_grad, bins, group, t, id_bits);
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
         fvec<D + 1> w;  // b_r * w_level (:405), or dB[r] * w_level (:1244-1245)
@@ -245,14 +246,14 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
             slot[r] = to_slot(h[r], capacity, cap_mask);
         });
         const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
-                                              streaming, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
+                                              mode, id_bits, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
         if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
         pos = pos_next;
         q = q_next;
         g0 = g0_next;
         g1 = g1_next;
     }
-    scatter_end(state, level_grad, bins, group, streaming);
+    scatter_end(state, level_grad, bins, group, mode, id_bits);
 }
 
 // ------------------------------------------------------------------------------------------

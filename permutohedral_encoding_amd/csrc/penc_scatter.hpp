@@ -14,6 +14,10 @@
 //   1. Accumulate cache in LDS.  Every workgroup keeps a small open-addressed table
 //      (tag = slot) for the level it works on.  Coarse levels, where thousands of points share
 //      a handful of vertices, are absorbed here completely; the table is flushed once at the end.
+//      When the first tile shows that the level has only a few dozen distinct slots, the cache's
+//      LDS is re-laid as one column of per-lane cells for each slot (column mode): lanes then
+//      add without meeting each other, and the wave-wide folding that a handful of hot lines
+//      needs, which is what bounds those levels (vector ALU), is not needed at all.
 //   2. Slot-range bins (optional, needs a workspace).  A contribution that finds no line in the
 //      cache is appended, as a 12-byte record, to the bin of its slot range (each workgroup has a
 //      private segment in every bin, so appending costs one LDS counter increment and one
@@ -51,7 +55,11 @@ constexpr int kCacheLinesLog2 = PENC_CACHE_LINES_LOG2;
 constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per workgroup
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
-constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space
+constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space or columns
+constexpr int kColumnMinIdsLog2 = 5;   // column mode: the cache's kCacheLines cells per feature are 32 columns of 64 cells (one per lane) ...
+constexpr int kColumnMaxIdsLog2 = 7;   // ... up to 128 columns of 16 cells, by the number of distinct slots the first tile has shown
+constexpr int kColumnProbes = 16;      // linear probes before a contribution gives up on the column table
+enum ScatterMode : int { kModeCache = 0, kModeStream = 1, kModeColumns = 2 };
 // vertices per thread a wave sorts by bin in one go (256 or 320 records): all D+1 of them up to D = 4
 constexpr int stage_chunk(int pos_dim) { return pos_dim + 1 <= 4 ? 4 : 5; }
 constexpr int kStageBins = 64;         // a wave counts one bin per lane: staging needs n_bins <= 64
@@ -188,6 +196,7 @@ struct ScatterStateT {
     uint4 stage_tail[kTail > 0 ? kTail : 1];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
     uint32_t hits;                 // contributions the cache has absorbed into existing lines
+    uint32_t lines;                // lines in use when the workgroup decided how to go on (see scatter_mode_switch)
 };
 
 template <typename State>
@@ -198,7 +207,10 @@ __device__ __forceinline__ void scatter_begin(State& c) {
         c.val[1][e] = 0.0;
     }
     for (int b = threadIdx.x; b < kMaxBins; b += kScatterBlock) c.bin_count[b] = 0u;
-    if (threadIdx.x == 0) c.hits = 0u;
+    if (threadIdx.x == 0) {
+        c.hits = 0u;
+        c.lines = 0u;
+    }
     __syncthreads();
 }
 
@@ -366,17 +378,97 @@ __device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_gra
     });
 }
 
+// Column mode of stage 1, for a level whose points share a few dozen slots.  The cache's values
+// are re-laid as 2^id_bits columns of kCacheLines >> id_bits cells; a slot owns a column (found
+// through the first 2^id_bits tags, open addressing with linear probing) and a lane adds into the
+// cell (lane mod cells) of its slot's column.  With 64 cells a lane meets no other lane of its
+// wave, whatever the slots; with 32 or 16 cells two or four lanes share a cell.  The columns are
+// summed when the level ends (column_flush).  Returns the column of `slot`, or -1 when the probes
+// find only other slots (the contribution then takes stage 2 or 3 like any miss).
+template <typename State>
+__device__ __forceinline__ int column_find(State& c, uint32_t slot, uint32_t id_bits) {
+    const int want = static_cast<int>(slot);
+    const uint32_t mask = (1u << id_bits) - 1u;
+    uint32_t e = (slot * 0x9E3779B1u) >> (32 - id_bits);
+#pragma unroll 1
+    for (int probe = 0; probe < kColumnProbes; ++probe) {
+        int owner = c.tag[e];
+        if (owner == want) return static_cast<int>(e);
+        if (owner == -1) {
+            owner = atomicCAS(&c.tag[e], -1, want);
+            if (owner == -1 || owner == want) return static_cast<int>(e);
+        }
+        e = (e + 1u) & mask;
+    }
+    return -1;
+}
+
+template <int D, typename State>
+__device__ __forceinline__ void column_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
+                                            uint32_t group, bool active, uint32_t id_bits, uvec<D + 1> slot,
+                                            fvec<D + 1> a0, fvec<D + 1> a1) {
+    const uint32_t cell_bits = kCacheLinesLog2 - id_bits;
+    const uint32_t my_cell = threadIdx.x & ((1u << cell_bits) - 1u);
+    static_for<D + 1>(PENC_BODY(r) {
+        PENC_INDEX(r);
+        bool miss = active;
+        if (active) {
+            const int e = column_find(c, slot[r], id_bits);
+            if (e >= 0) {
+                const uint32_t cell = (static_cast<uint32_t>(e) << cell_bits) | my_cell;
+                __hip_atomic_fetch_add(&c.val[0][cell], static_cast<double>(a0[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&c.val[1][cell], static_cast<double>(a1[r]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                miss = false;
+            }
+        }
+        if (miss && bins.records != nullptr) miss = !append_record(c, bins, group, slot[r], a0[r], a1[r]);
+        if (__any(miss)) global_add_pairs(level_grad, miss, slot[r], a0[r], a1[r]);
+    });
+}
+
+// Sums every column in use and sends the sums on to stage 2 (or 3).  By all threads, between barriers.
+template <typename State>
+__device__ __forceinline__ void column_flush(State& c, const GradSlice& level_grad, const BinTarget& bins,
+                                             uint32_t group, uint32_t id_bits) {
+    const uint32_t cell_bits = kCacheLinesLog2 - id_bits, cells = 1u << cell_bits;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (uint32_t id = wave; id < (1u << id_bits); id += kScatterBlock / 64) {
+        const int owner = c.tag[id];  // the same for all lanes of the wave
+        if (owner == -1) continue;
+        double s0 = lane < cells ? c.val[0][(id << cell_bits) + lane] : 0.0;
+        double s1 = lane < cells ? c.val[1][(id << cell_bits) + lane] : 0.0;
+#pragma unroll
+        for (int step = 32; step > 0; step >>= 1) {
+            s0 += __shfl_xor(s0, step);
+            s1 += __shfl_xor(s1, step);
+        }
+        if (lane == 0) {
+            const float v0 = static_cast<float>(s0), v1 = static_cast<float>(s1);
+            const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
+            if (!binned) {
+                float* g = level_grad.at(static_cast<uint32_t>(owner));
+                global_add(g, v0);
+                global_add(g + 1, v1);
+            }
+        }
+    }
+}
+
 // One tile's D+1 contributions per thread through stages 1-3.  All 64 lanes of every wave must
 // call it together; `active` is false for lanes that carry no point (tail of the last tile), which
 // only take part in the wave-wide steps.  `use_cache` (wave-uniform) is false once the workgroup
-// has seen that the cache does not hit at this level; `streaming` is what scatter_stream_switch
-// returned.  The return value is the number of hits of this wave in this tile.
+// has seen that the cache does not hit at this level; `mode` and `id_bits` are what
+// scatter_mode_switch decided.  The return value is the number of hits of this wave in this tile.
 template <int D, typename State>
 __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
-                                                 uint32_t group, bool active, bool use_cache, bool streaming,
+                                                 uint32_t group, bool active, bool use_cache, int mode, uint32_t id_bits,
                                                  uvec<D + 1> slot, fvec<D + 1> a0, fvec<D + 1> a1) {
-    if (streaming) {
+    if (mode == kModeStream) {
         stream_tile<D>(c, level_grad, bins, group, active, slot, a0, a1);
+        return 0u;
+    }
+    if (mode == kModeColumns) {
+        column_tile<D>(c, level_grad, bins, group, active, id_bits, slot, a0, a1);
         return 0u;
     }
     uint32_t hits = 0;
@@ -450,30 +542,53 @@ __device__ __forceinline__ void cache_flush(State& c, const GradSlice& level_gra
     }
 }
 
-// Before tile `tile` (all threads call it, with the same arguments): decides for the whole
-// workgroup whether to give up the accumulate cache for good and use its LDS as staging space
-// (stream_tile).  Returns true from then on; the cache's contents have been flushed by then.
+// Before tile kStreamDecisionTile (all threads call it, with the same arguments): decides for the
+// whole workgroup how the rest of the level goes.  A cache that does not hit is given up for good
+// and its LDS becomes staging space (kModeStream, see stream_tile; needs bins); a cache that hits
+// on at most 64 lines becomes columns (kModeColumns, `id_bits` says how many); otherwise the
+// cache stays.  On a change of mode the cache's contents have been flushed on return.
 template <int D, typename State>
-__device__ __forceinline__ bool scatter_stream_switch(State& c, const GradSlice& level_grad,
-                                                      const BinTarget& bins, uint32_t group, int tile) {
-    if (tile != kStreamDecisionTile || bins.records == nullptr || bins.n_bins > kStageBins) return false;
+__device__ __forceinline__ int scatter_mode_switch(State& c, const GradSlice& level_grad, const BinTarget& bins,
+                                                   uint32_t group, int tile, uint32_t& id_bits) {
     __syncthreads();  // the hits of the tiles so far are in
-    const bool stream = !cache_pays<D>(c, tile);
-    __syncthreads();  // everyone has read the count before a fast wave adds the next tile's hits
-    if (!stream) return false;
+    const bool pays = cache_pays<D>(c, tile);
+    if (pays) {
+        uint32_t used = 0;
+        for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) used += __popcll(__ballot(c.tag[e] != -1));
+        if ((threadIdx.x & 63) == 0 && used != 0u) atomicAdd(&c.lines, used);
+    }
+    __syncthreads();  // everyone has read the hits before a fast wave adds the next tile's; the line count is in
+    int mode = kModeCache;
+    if (!pays) {
+        if (bins.records != nullptr && bins.n_bins <= kStageBins) mode = kModeStream;
+    } else if (c.lines <= (1u << (kColumnMaxIdsLog2 - 1))) {  // the table of columns stays at most half full
+        mode = kModeColumns;
+        id_bits = kColumnMinIdsLog2;
+        while ((1u << (id_bits - 1)) < c.lines) ++id_bits;
+    }
+    if (mode == kModeCache) return mode;
     cache_flush(c, level_grad, bins, group);
     __syncthreads();
-    return true;
+    if (mode == kModeColumns) {
+        for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
+            c.tag[e] = -1;
+            c.val[0][e] = 0.0;
+            c.val[1][e] = 0.0;
+        }
+        __syncthreads();
+    }
+    return mode;
 }
 
-// After the last tile: flushes the accumulate cache (through the bins when there are any; a
-// streaming workgroup has none left) and publishes how many records this workgroup left in each
+// After the last tile: flushes the accumulate cache or the columns (through the bins when there are
+// any; a streaming workgroup has neither left) and publishes how many records this workgroup left in each
 // bin.  Call once, by all threads.
 template <typename State>
 __device__ __forceinline__ void scatter_end(State& c, const GradSlice& level_grad, const BinTarget& bins,
-                                            uint32_t group, bool streaming) {
+                                            uint32_t group, int mode, uint32_t id_bits) {
     __syncthreads();
-    if (!streaming) cache_flush(c, level_grad, bins, group);
+    if (mode == kModeCache) cache_flush(c, level_grad, bins, group);
+    if (mode == kModeColumns) column_flush(c, level_grad, bins, group, id_bits);
     if (bins.records == nullptr) return;
     __syncthreads();
     for (uint32_t b = threadIdx.x; b < bins.n_bins; b += kScatterBlock) {
