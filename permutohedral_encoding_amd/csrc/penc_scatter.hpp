@@ -25,8 +25,8 @@
 //      LDS (fp64), and adds the range into the gradient with coalesced read-modify-writes.  This
 //      turns the random scatter of the fine levels into streaming traffic.  Once a workgroup has
 //      seen that its cache does not hit at a level, it gives the cache's LDS to its wavefronts as
-//      staging space: each wave sorts the records of a tile by bin there, so that records of one
-//      bin leave in runs of consecutive addresses instead of one 12-byte store each.
+//      staging space: the workgroup sorts the records of a tile by bin there, so that records of one
+//      bin leave in runs of consecutive addresses (whole cache lines) instead of one 12-byte store each.
 //   3. Direct global atomics, with the two features of a slot in one instruction (lane pairs),
 //      for whatever is left: no workspace, capacity too large for binning, or a full bin.
 // The result never depends on a stage hitting: every stage falls through to the next.
@@ -258,8 +258,127 @@ __device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) 
     return -1;
 }
 
-// Stage 2 for a whole tile once the workgroup streams (see scatter_stream_switch): the cache's LDS
-// is staging space, a 4 or 5 KiB slice per wave.  For stage_chunk(D) vertices per thread at a time, the wave
+// Stage 2 for a whole tile once the workgroup streams (see scatter_mode_switch): the cache's LDS is
+// staging space for a counting sort of the tile's records by bin, stage_chunk(D) vertices per thread
+// at a time (2048 or 2560 records).  Every wave counts its records per bin (one LDS counter per
+// bin and wave); the first wave turns the counts into run offsets (a bin's run is the waves' runs
+// one after the other) and reserves room for each bin's run in the workgroup's segment with one
+// add per bin; the waves lay their records out in that order in the staging space; and then all
+// threads store the records in staging order: a wave instruction writes 64 consecutive records
+// of (mostly) one bin, i.e. whole cache lines, where the records of a single wave would leave in
+// runs of eight.  A staged record carries its destination (its index in the level's record
+// array), so the store needs no search.  When a run does not fit its segment any more (rare: the
+// segments hold the mean plus three standard deviations) the chunk checks every record against
+// the room left and sends the excess to stage 3.
+// Needs bins.n_bins <= kStageBins and a level's record array below 2^32 bytes (the host plans
+// for both); all threads of the workgroup must call it together.
+template <int D, typename State>
+__device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
+                                            uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
+                                            fvec<D + 1> a1) {
+    constexpr int kWaves = kScatterBlock / 64;
+    constexpr int kStageChunk = State::kChunk;
+    static_assert(kCacheLines >= (3 * kWaves + 3) * 64, "the sort's index arrays live in the tag array");
+    static_assert(offsetof(State, stage_tail) == offsetof(State, val) + sizeof(c.val) &&
+                      (sizeof(c.val) + (State::kTail > 0 ? sizeof(c.stage_tail) : 0)) == kStageChunk * kScatterBlock * sizeof(uint4),
+                  "val and stage_tail are one contiguous staging array");
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    uint32_t* const words = reinterpret_cast<uint32_t*>(c.tag);
+    uint32_t* const count = words + wave * 64;                  // [wave][bin] records of this wave per bin
+    uint32_t* const offset = words + (kWaves + wave) * 64;      // [wave][bin] where the wave's run starts in the staging array
+    uint32_t* const dest = words + (2 * kWaves + wave) * 64;    // [wave][bin] index of the run's first record in the level's record array
+    uint32_t* const run_first = words + 3 * kWaves * 64;        // [bin] index of the workgroup's run for the bin
+    uint32_t* const room = run_first + 64;                      // [bin] records the workgroup's segment can still take
+    uint32_t* const header = room + 64;                         // [0] records staged, [1] whether every run fits
+    uint4* const stage = reinterpret_cast<uint4*>(c.val);
+    char* const record_bytes = reinterpret_cast<char*>(bins.records);
+    constexpr uint32_t kNoRoom = 0xFFFFFFFFu;
+    constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
+    static_for<kChunks>(PENC_BODY(chunk) {
+        PENC_INDEX(chunk);
+        constexpr int kFirst = chunk * kStageChunk;
+        constexpr int kCount = D + 1 - kFirst < kStageChunk ? D + 1 - kFirst : kStageChunk;
+        count[lane] = 0u;
+        wave_lds_fence();
+        uvec<kStageChunk> place = 0u;  // rank of each record within its wave's run for the bin
+        static_for<kCount>(PENC_BODY(j) {
+            PENC_INDEX(j);
+            if (active) place[j] = atomicAdd(&count[slot[kFirst + j] >> kBinSlotsLog2], 1u);
+        });
+        __syncthreads();
+        if (wave == 0) {  // lane b looks after bin b
+            uint32_t before[kWaves], mine = 0u;
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                before[w] = mine;
+                mine += words[w * 64 + lane];
+            }
+            uint32_t total;
+            const uint32_t first = wave_exclusive_scan(mine, total);
+            const uint32_t taken = mine != 0u ? atomicAdd(&c.bin_count[lane], mine) : 0u;
+            const uint32_t start = (lane * bins.n_groups + group) * bins.segment_capacity + taken;
+            const bool all_fit = __all(taken + mine <= bins.segment_capacity);
+#pragma unroll
+            for (int w = 0; w < kWaves; ++w) {
+                words[(kWaves + w) * 64 + lane] = first + before[w];
+                words[(2 * kWaves + w) * 64 + lane] = start + before[w];
+            }
+            run_first[lane] = start;
+            room[lane] = taken < bins.segment_capacity ? bins.segment_capacity - taken : 0u;
+            if (lane == 0) {
+                header[0] = total;
+                header[1] = all_fit ? 1u : 0u;
+            }
+        }
+        __syncthreads();
+        const uint32_t total = header[0];
+        const bool all_fit = header[1] != 0u;
+        static_for<kCount>(PENC_BODY(j) {
+            PENC_INDEX(j);
+            if (active) {
+                const uint32_t b = slot[kFirst + j] >> kBinSlotsLog2;
+                // copies first: a bit cast applied directly to a vector element reads element 0
+                const float v0 = a0[kFirst + j], v1 = a1[kFirst + j];
+                const uint32_t to = dest[b] + place[j];
+                uint4 e;
+                e.x = slot[kFirst + j];
+                e.y = __builtin_bit_cast(uint32_t, v0);
+                e.z = __builtin_bit_cast(uint32_t, v1);
+                e.w = all_fit || to - run_first[b] < room[b] ? to : kNoRoom;
+                stage[offset[b] + place[j]] = e;
+            }
+        });
+        __syncthreads();
+        static_for<kCount>(PENC_BODY(j) {
+            PENC_INDEX(j);
+            const uint32_t i = j * kScatterBlock + threadIdx.x;
+            bool spill = false;
+            uint4 e = {0u, 0u, 0u, 0u};
+            if (i < total) {
+                e = stage[i];
+                if (e.w != kNoRoom) {
+                    BinRecord rec;
+                    rec.slot_in_bin = e.x & (kBinSlots - 1);
+                    rec.a0 = __builtin_bit_cast(float, e.y);
+                    rec.a1 = __builtin_bit_cast(float, e.z);
+                    *reinterpret_cast<BinRecord*>(record_bytes + e.w * static_cast<uint32_t>(sizeof(BinRecord))) = rec;
+                } else {
+                    spill = true;  // the segment is full: stage 3
+                }
+            }
+            if (!all_fit && __any(spill))
+                global_add_pairs(level_grad, spill, e.x, __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
+        });
+        // the next chunk (or tile) writes the counters after this wave's loads above and the staging
+        // array after its next two barriers: nothing here is overwritten while another wave reads it
+        wave_lds_fence();
+    });
+}
+
+// The same sort with every wave on its own (no barriers), for the dimensions whose D+1 vertices
+// take two chunks: the waves of a workgroup drift apart over their longer tiles, and waiting for
+// each other three times per chunk then costs more than the longer runs save (measured at D = 8).
+// The staging space is a 4 or 5 KiB slice per wave.  For stage_chunk(D) vertices per thread at a time, the wave
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
 // its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
@@ -270,7 +389,7 @@ __device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) 
 // Needs bins.n_bins <= kStageBins and a level's record array below 2^32 bytes (the host plans
 // for both); all 64 lanes of the wave must call it together.
 template <int D, typename State>
-__device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
+__device__ __forceinline__ void stream_tile_wave(State& c, const GradSlice& level_grad, const BinTarget& bins,
                                             uint32_t group, bool active, uvec<D + 1> slot, fvec<D + 1> a0,
                                             fvec<D + 1> a1) {
     constexpr int kWaves = kScatterBlock / 64;
@@ -464,7 +583,11 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
                                                  uint32_t group, bool active, bool use_cache, int mode, uint32_t id_bits,
                                                  uvec<D + 1> slot, fvec<D + 1> a0, fvec<D + 1> a1) {
     if (mode == kModeStream) {
-        stream_tile<D>(c, level_grad, bins, group, active, slot, a0, a1);
+        if constexpr (D + 1 <= State::kChunk) {
+            stream_tile<D>(c, level_grad, bins, group, active, slot, a0, a1);
+        } else {
+            stream_tile_wave<D>(c, level_grad, bins, group, active, slot, a0, a1);
+        }
         return 0u;
     }
     if (mode == kModeColumns) {
