@@ -231,7 +231,6 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
                 out[n_points] = g1;
             }
         }
-        if (t == kStreamDecisionTile) mode = scatter_mode_switch<D>(state, level_grad, bins, group, t, id_bits);
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
         fvec<D + 1> w;  // b_r * w_level (:405), or dB[r] * w_level (:1244-1245)
@@ -245,9 +244,11 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
             PENC_INDEX(r);
             slot[r] = to_slot(h[r], capacity, cap_mask);
         });
+        if (t == 0) mode = scatter_mode_decide<D>(state, bins, active, slot, id_bits);
         const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
                                               mode, id_bits, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
-        if ((threadIdx.x & 63) == 0 && hits) atomicAdd(&state.hits, hits);
+        // the first tile finds the lines its own look-up has claimed: no evidence of reuse
+        if ((threadIdx.x & 63) == 0 && hits && t > 0) atomicAdd(&state.hits, hits);
         pos = pos_next;
         q = q_next;
         g0 = g0_next;

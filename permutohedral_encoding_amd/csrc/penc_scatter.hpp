@@ -55,7 +55,6 @@ constexpr int kCacheLinesLog2 = PENC_CACHE_LINES_LOG2;
 constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per workgroup
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
-constexpr int kStreamDecisionTile = 1; // tile before which a workgroup may turn its cache into staging space or columns
 constexpr int kColumnMinIdsLog2 = 5;   // column mode: the cache's kCacheLines cells per feature are 32 columns of 64 cells (one per lane) ...
 constexpr int kColumnMaxIdsLog2 = 7;   // ... up to 128 columns of 16 cells, by the number of distinct slots the first tile has shown
 constexpr int kColumnProbes = 16;      // linear probes before a contribution gives up on the column table
@@ -195,8 +194,11 @@ struct ScatterStateT {
     // when the workgroup streams, val and this tail together are its waves' staging slices
     uint4 stage_tail[kTail > 0 ? kTail : 1];
     uint32_t bin_count[kMaxBins];  // records this workgroup has appended to each bin so far
-    uint32_t hits;                 // contributions the cache has absorbed into existing lines
-    uint32_t lines;                // lines in use when the workgroup decided how to go on (see scatter_mode_switch)
+    uint32_t hits;                 // contributions the cache has absorbed into existing lines since the first tile
+    // what the look-ups of the first tile's slots showed (see scatter_mode_decide)
+    uint32_t wanted;               // contributions of the first tile
+    uint32_t lines;                // lines they claimed: the tile's distinct slots, as far as the cache could take them
+    uint32_t misses;               // contributions whose slot found no line
 };
 
 template <typename State>
@@ -209,7 +211,9 @@ __device__ __forceinline__ void scatter_begin(State& c) {
     for (int b = threadIdx.x; b < kMaxBins; b += kScatterBlock) c.bin_count[b] = 0u;
     if (threadIdx.x == 0) {
         c.hits = 0u;
+        c.wanted = 0u;
         c.lines = 0u;
+        c.misses = 0u;
     }
     __syncthreads();
 }
@@ -258,7 +262,7 @@ __device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) 
     return -1;
 }
 
-// Stage 2 for a whole tile once the workgroup streams (see scatter_mode_switch): the cache's LDS is
+// Stage 2 for a whole tile once the workgroup streams (see scatter_mode_decide): the cache's LDS is
 // staging space for a counting sort of the tile's records by bin, stage_chunk(D) vertices per thread
 // at a time (2048 or 2560 records).  Every wave counts its records per bin (one LDS counter per
 // bin and wave); the first wave turns the counts into run offsets (a bin's run is the waves' runs
@@ -577,7 +581,7 @@ __device__ __forceinline__ void column_flush(State& c, const GradSlice& level_gr
 // call it together; `active` is false for lanes that carry no point (tail of the last tile), which
 // only take part in the wave-wide steps.  `use_cache` (wave-uniform) is false once the workgroup
 // has seen that the cache does not hit at this level; `mode` and `id_bits` are what
-// scatter_mode_switch decided.  The return value is the number of hits of this wave in this tile.
+// scatter_mode_decide decided.  The return value is the number of hits of this wave in this tile.
 template <int D, typename State>
 __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& level_grad, const BinTarget& bins,
                                                  uint32_t group, bool active, bool use_cache, int mode, uint32_t id_bits,
@@ -640,11 +644,18 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
     return hits;
 }
 
-// The workgroup-wide decision whether stage 1 is worth its LDS traffic at this level: after the
-// first tile, keep using the cache only while at least one contribution in eight hits.
+// The workgroup-wide decision whether stage 1 is worth its LDS traffic at this level: keep using the
+// cache only while at least one contribution in `one_in` hits.  The evidence before tile `tile` is
+// the look-up of the first tile's slots (a contribution that neither claimed a line nor missed
+// would have hit) and the hits of the tiles processed since.  Against appending every miss to its
+// bin on its own, one hit in eight pays; against sorting the tile's records by bin (stream_tile),
+// which is cheaper than the cache's look-ups, it takes one in four.
 template <int D, typename State>
-__device__ __forceinline__ bool cache_pays(const State& c, int tiles_done) {
-    return tiles_done == 0 || c.hits * 8u >= static_cast<uint32_t>(tiles_done) * kScatterBlock * (D + 1);
+__device__ __forceinline__ bool cache_pays(const State& c, int tile, uint32_t one_in = 8u) {
+    const uint32_t settled = c.lines + c.misses;
+    const uint32_t first_hits = c.wanted > settled ? c.wanted - settled : 0u;
+    const uint32_t seen = c.wanted + static_cast<uint32_t>(tile > 1 ? tile - 1 : 0) * kScatterBlock * (D + 1);
+    return (first_hits + c.hits) * one_in >= seen;
 }
 
 // Sends every line of the accumulate cache on to stage 2 (or 3).  By all threads, between barriers.
@@ -665,39 +676,41 @@ __device__ __forceinline__ void cache_flush(State& c, const GradSlice& level_gra
     }
 }
 
-// Before tile kStreamDecisionTile (all threads call it, with the same arguments): decides for the
-// whole workgroup how the rest of the level goes.  A cache that does not hit is given up for good
-// and its LDS becomes staging space (kModeStream, see stream_tile; needs bins); a cache that hits
-// on at most 64 lines becomes columns (kModeColumns, `id_bits` says how many); otherwise the
-// cache stays.  On a change of mode the cache's contents have been flushed on return.
+// Before the first tile is scattered (all threads call it, with the tile's slots): decides for the
+// whole workgroup how the level goes.  The slots are looked up in the (empty) cache, which claims a
+// line for every distinct slot as far as it can; the counts tell what the cache is good for.  One
+// that would not hit is never filled: its LDS becomes staging space (kModeStream, see
+// stream_tile; needs bins).  One that hits on at most 64 lines becomes columns (kModeColumns,
+// `id_bits` says how many).  Otherwise the cache serves, with the lines already claimed.
 template <int D, typename State>
-__device__ __forceinline__ int scatter_mode_switch(State& c, const GradSlice& level_grad, const BinTarget& bins,
-                                                   uint32_t group, int tile, uint32_t& id_bits) {
-    __syncthreads();  // the hits of the tiles so far are in
-    const bool pays = cache_pays<D>(c, tile);
-    if (pays) {
-        uint32_t used = 0;
-        for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) used += __popcll(__ballot(c.tag[e] != -1));
-        if ((threadIdx.x & 63) == 0 && used != 0u) atomicAdd(&c.lines, used);
+__device__ __forceinline__ int scatter_mode_decide(State& c, const BinTarget& bins, bool active, uvec<D + 1> slot,
+                                                   uint32_t& id_bits) {
+    uint32_t wanted = 0, missed = 0;  // over the wave
+    static_for<D + 1>(PENC_BODY(r) {
+        PENC_INDEX(r);
+        bool found = false;
+        const bool miss = active && cache_find(c, slot[r], found) < 0;
+        wanted += __popcll(__ballot(active));
+        missed += __popcll(__ballot(miss));
+    });
+    if ((threadIdx.x & 63) == 0) {
+        atomicAdd(&c.wanted, wanted);
+        if (missed != 0u) atomicAdd(&c.misses, missed);
     }
-    __syncthreads();  // everyone has read the hits before a fast wave adds the next tile's; the line count is in
+    __syncthreads();  // every line the tile wants is claimed
+    uint32_t used = 0;
+    for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) used += __popcll(__ballot(c.tag[e] != -1));
+    if ((threadIdx.x & 63) == 0 && used != 0u) atomicAdd(&c.lines, used);
+    __syncthreads();
     int mode = kModeCache;
-    if (!pays) {
-        if (bins.records != nullptr && bins.n_bins <= kStageBins) mode = kModeStream;
-    } else if (c.lines <= (1u << (kColumnMaxIdsLog2 - 1))) {  // the table of columns stays at most half full
+    const bool can_stream = bins.records != nullptr && bins.n_bins <= kStageBins;
+    if (can_stream && !cache_pays<D>(c, 0, 4u)) {
+        mode = kModeStream;
+    } else if (cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1))) {  // the table of columns starts at most half full
         mode = kModeColumns;
         id_bits = kColumnMinIdsLog2;
         while ((1u << (id_bits - 1)) < c.lines) ++id_bits;
-    }
-    if (mode == kModeCache) return mode;
-    cache_flush(c, level_grad, bins, group);
-    __syncthreads();
-    if (mode == kModeColumns) {
-        for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) {
-            c.tag[e] = -1;
-            c.val[0][e] = 0.0;
-            c.val[1][e] = 0.0;
-        }
+        for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) c.tag[e] = -1;  // now the table of columns
         __syncthreads();
     }
     return mode;
