@@ -608,6 +608,54 @@ def test_many_bins_and_few_contributions_per_slot():
         assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, {n} points")
 
 
+def _table_gradients_match(p, d, cap, what):
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"])
+    inp = gpu_input(p, need_pos_grad=False)
+    tg, _ = enc.backward(inp, to_gpu(p["grad"]))
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, what + ", table gradient")
+    tg2, _ = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, what + ", second-order table gradient")
+
+
+@pytest.mark.parametrize("d", [3, 4, 6])
+def test_first_tile_misleads_the_scatter_about_the_level(d):
+    """A scattering workgroup chooses how it accumulates a level (a column of cells per slot, the
+    accumulate cache, or records sorted by bin) from the first 512 of its 4096 or 8192 points.  Points
+    laid out so that the choice is wrong for the rest of the group: (a) the first 512 points of every
+    group sit in one simplex at every level and the others are spread out, so the few columns overflow
+    and the rest goes to bins or atomics contribution by contribution; (b) the first 512 are spread out
+    and all the others sit in one simplex, so the sorted stream sends thousands of records to the
+    same few bins and their segments overflow into direct atomics."""
+    n, levels, cap = 3 * 8192 + 777, 6, 1 << 15
+    rng = np.random.default_rng(90 + d)
+    first_tile = (np.arange(n) % 4096) < 512
+    cluster = (0.37 + 1e-7 * rng.standard_normal((n, d))).astype(np.float32)
+    for what, clustered in (("columns overflow", first_tile), ("segments overflow", ~first_tile)):
+        p = random_problem(d, n, levels, cap, seed=91 + d, sigma_range=(1.0, 1e-3))
+        p["pos"] = np.where(clustered[:, None], cluster, p["pos"]).astype(np.float32)
+        _table_gradients_match(p, d, cap, what)
+
+
+def test_records_crowd_one_bin():
+    """Points chosen so that, at the finest level, at least three of their four vertices fall into the
+    first of four slot ranges: the tile's records are all distinct (the workgroup streams them sorted
+    by bin) but one bin receives three quarters of them where its segments are sized for a quarter plus
+    three standard deviations, so most chunks take the path that checks every record against the room
+    left and spills the excess."""
+    d, levels, cap = 3, 3, 1 << 15
+    p = random_problem(d, 600000, levels, cap, seed=97, sigma_range=(1e-2, 1e-3))
+    sf = orc.scale_factors(d, p["sigmas"])
+    slots = orc.simplex(p["pos"], sf, p["shift"], cap)["slot"][levels - 1]  # (N, D+1)
+    crowded = np.sum(slots < (1 << 13), axis=1) >= 3
+    keep = np.flatnonzero(crowded)[:20000]
+    assert len(keep) >= 18000
+    p["pos"], p["dpos"], p["grad"] = p["pos"][keep], p["dpos"][keep], np.ascontiguousarray(p["grad"][:, :, keep])
+    _table_gradients_match(p, d, cap, "one crowded bin")
+
+
 @pytest.mark.parametrize("d", [2, 5, 6, 7])
 def test_large_size_identities_in_the_other_dimensions(d):
     """The benchmark configurations cover D = 3, 4, 8 at full size; the same size-independent checks for
