@@ -149,7 +149,7 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
 // is [L * F/2][2][N], and in a row the pair sits at column 2 * pair_level.
 template <int D, bool kRowMajor, bool kSecondOrder>
 __global__ void __launch_bounds__(kScatterBlock)
-backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t feat_pairs, int tiles_per_group,
+backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t feat_pairs, uint32_t dies, int tiles_per_group,
                       uint32_t capacity, uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
                       const float* __restrict__ random_shift, const float* __restrict__ window,
@@ -157,14 +157,14 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
                       const float* __restrict__ double_pos_grad, float* __restrict__ table_grad,
                       float* __restrict__ grad_level_major, BinTarget pass_bins) {
     __shared__ ScatterStateT<stage_chunk(D)> state;
-    // Workgroups are dealt round-robin to the kXcds dies, each with an L2 of its own.  The j-th
+    // Workgroups are dealt round-robin to the chip's `dies` dies, each with an L2 of its own.  The j-th
     // workgroup of a die takes level j % levels of one group of points: a die works through all
     // levels of a group before the next group, so the points are fetched from memory once, and
     // compute-bound coarse levels and store-bound fine levels share the chip at all times (this
     // kernel never reads the table: there is no slice to keep cache-resident by running a level at
     // a time).
-    const uint32_t die = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
-    const uint32_t level_in_pass = j % n_pass_levels, group = (j / n_pass_levels) * kXcds + die;
+    const uint32_t die = blockIdx.x % dies, j = blockIdx.x / dies;
+    const uint32_t level_in_pass = j % n_pass_levels, group = (j / n_pass_levels) * dies + die;
     const int64_t group_base = static_cast<int64_t>(group) * tiles_per_group * kScatterBlock;
     if (group_base >= n_points) return;
     const uint32_t pair_level = static_cast<uint32_t>(first_level) + level_in_pass;
@@ -628,6 +628,25 @@ inline void* static_scratch_of_current_device() {
     return address[device];
 }
 
+// Accelerator dies of the current GPU (each with an L2 of its own; workgroup i of a launch runs on
+// die i % dies), asked of the runtime once per device.  kDefaultDies when the runtime does not say.
+inline uint32_t dies_of_current_device() {
+    static std::mutex lock;
+    static uint32_t dies[kMaxDevices] = {};
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return kDefaultDies;
+    std::lock_guard<std::mutex> guard(lock);
+    if (dies[device] == 0u) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeNumberOfXccs, device) != hipSuccess) {
+            (void)hipGetLastError();
+            n = 0;
+        }
+        dies[device] = n >= 1 && n <= 64 ? static_cast<uint32_t>(n) : kDefaultDies;
+    }
+    return dies[device];
+}
+
 }  // namespace penc
 
 using namespace penc;
@@ -651,14 +670,15 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
     const int tiles_per_group = table_backward_tiles(nr_positions, pair_levels);
     const BinPlan plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
     const int per_pass = plan.enabled ? plan.levels_per_pass : pair_levels;
+    const uint32_t dies = dies_of_current_device();
     for (int first = 0; first < pair_levels; first += per_pass) {
         const int count = pair_levels - first < per_pass ? pair_levels - first : per_pass;
-        const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + kXcds - 1) / kXcds * kXcds;
+        const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + dies - 1) / dies * dies;
         const dim3 grid(padded_groups * static_cast<unsigned>(count));
 #define PENC_LAUNCH_TABLE(ROW_MAJOR, SECOND_ORDER)                                                                         \
     PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER>), grid,                  \
                                                 dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
-                                                feat_pairs, tiles_per_group, cap, mask, positions, scale_factor,             \
+                                                feat_pairs, dies, tiles_per_group, cap, mask, positions, scale_factor,       \
                                                 random_shift, anneal_window, grad, grad_row_stride, double_pos_grad,         \
                                                 lattice_values_grad, grad_level_major, plan.target))
         if (double_pos_grad != nullptr && grad_row_stride != 0) {

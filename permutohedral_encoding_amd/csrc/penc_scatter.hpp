@@ -40,7 +40,7 @@
 
 namespace penc {
 
-constexpr int kXcds = 8;               // accelerator dies (XCDs) of the chip; workgroup i runs on die i % kXcds
+constexpr uint32_t kDefaultDies = 8;   // accelerator dies (XCDs) of an MI355X, for when the runtime does not tell
 constexpr int kBlock = 256;            // threads per workgroup of the gather-type kernels (4 wavefronts)
 #ifndef PENC_SCATTER_BLOCK
 #define PENC_SCATTER_BLOCK 512
