@@ -13,7 +13,8 @@
  *    the enqueued work.  The library never allocates or frees device memory and keeps no state.
  *  - All arrays are fp32, densely packed, row-major (F = nr_feat, the features per level: 2, 4 or 8):
  *        positions            [N][D]
- *        lattice_values       [L][C][F]      (8-byte aligned for F = 2, 16-byte for F = 4 and 8)
+ *        lattice_values       [L][C][F]      (8-byte aligned for F = 2, 16-byte for F = 4 and 8;
+ *                                            binary16 in the *_half entry points)
  *        scale_factor         [L][D]         (from penc_scale_factors)
  *        random_shift         [L][D]
  *        anneal_window        [L]
@@ -183,6 +184,33 @@ int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64
                                                  float* lattice_values_grad, float* grad_grad_sliced_values,
                                                  int concat_points, void* workspace, size_t workspace_bytes,
                                                  void* stream);
+
+/* The three gathering entry points for a table kept in half precision: lattice_values_half is
+ * [L][C][F] of IEEE binary16 (aligned to one slot of 2F bytes).  The values are widened exactly
+ * on load and all arithmetic stays fp32, so the results are those of the fp32 entry points on the
+ * widened table; sliced values, both gradients and grad_grad_sliced_values are fp32 as before (the
+ * table gradient never reads the table).  grad_row_stride selects the layout of the upstream
+ * gradient: 0 for [L+E][F][N], otherwise rows of that many floats as in the *_rowmajor entry points
+ * (with their workspace rules).
+ * Replaces: nothing that runs in the reference; it carries the intent as a disabled switch
+ * (LATTICE_HALF_PRECISION, kernels/permutohedral_encoding/EncodingGPU.cuh:12) beside the same
+ * forward / backward / double_backward_from_positions (src/Encoding.cu:55-334). */
+int penc_forward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                      const float* positions, const void* lattice_values_half, const float* scale_factor,
+                      const float* random_shift, const float* anneal_window, float* sliced_values,
+                      int concat_points, float points_scaling, void* stream);
+int penc_backward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                       const float* positions, const void* lattice_values_half, const float* scale_factor,
+                       const float* random_shift, const float* anneal_window, const float* grad,
+                       int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                       void* workspace, size_t workspace_bytes, void* stream);
+int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                             const float* positions, const void* lattice_values_half,
+                                             const float* scale_factor, const float* random_shift,
+                                             const float* anneal_window, const float* double_positions_grad,
+                                             const float* grad, int64_t grad_row_stride, float* lattice_values_grad,
+                                             float* grad_grad_sliced_values, int concat_points, void* workspace,
+                                             size_t workspace_bytes, void* stream);
 
 /* dst[c][r] = src[r][c] for a dense row-major rows x cols matrix with cols <= 255 (2 * levels):
  * turns the row-major upstream gradient (N, 2(L+E)) into the grad_sliced_values layout

@@ -53,6 +53,17 @@ _SIGNATURES = {
                                                            ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int,
                                                            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_forward_half": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                         _c_f32p, ctypes.c_void_p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                         ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
+    "penc_backward_half": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                          _c_f32p, ctypes.c_void_p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
+                                          _c_f32p, _c_f32p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_double_backward_from_positions_half": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                                                ctypes.c_int, _c_f32p, ctypes.c_void_p, _c_f32p, _c_f32p,
+                                                                _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
+                                                                _c_f32p, ctypes.c_int, ctypes.c_void_p,
+                                                                ctypes.c_size_t, ctypes.c_void_p]),
     "penc_transpose": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
                                           _c_f32p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -247,6 +258,21 @@ class EncodingWrapper:
         return EncodingWrapper(pos_dim, nr_feat_per_level, fixed_params)
 
     # -- checks shared by the three calls (reference: src/Encoding.cu:38-45, 57-66, 119-125)
+    half_table = False  # set by the module: gather from a half-precision copy of the fp32 table
+    _half_copy = None
+    _half_copy_of = None
+
+    def gather_table(self, lattice_values):
+        """The tensor the gathering kernels read for ``lattice_values``: the tensor itself, or, with
+        ``half_table``, its float16 copy, made again whenever the tensor has been modified in place."""
+        if not self.half_table or lattice_values.dtype != torch.float32:
+            return lattice_values
+        key = (lattice_values.data_ptr(), lattice_values._version, lattice_values.device, tuple(lattice_values.shape))
+        if self._half_copy_of != key:
+            self._half_copy = lattice_values.detach().to(torch.float16)
+            self._half_copy_of = key
+        return self._half_copy
+
     def _check_common(self, inp):
         fp = self.fixed_params
         pos, lv, win = inp.m_positions_raw, inp.m_lattice_values, inp.m_anneal_window
@@ -255,8 +281,12 @@ class EncodingWrapper:
         _require(pos.shape[1] == fp.m_pos_dim,
                  f"Pos dim for the lattice doesn't correspond with the position of the points. Lattice was initialized "
                  f"with {fp.m_pos_dim} and points have pos dim {pos.shape[1]}")
-        _check_f32_gpu(lv, "lattice_values", 3)
-        _require(lv.is_contiguous(), "lattice_values must be contiguous (two floats are loaded at a time)")
+        if isinstance(lv, torch.Tensor) and lv.dtype == torch.float16:  # a table kept in half precision: the *_half entry points
+            _require(lv.is_cuda, "lattice_values should be in GPU memory. Please call .cuda() on the tensor")
+            _require(lv.dim() == 3, f"lattice_values should have 3 dimensions, however it has sizes {tuple(lv.shape)}")
+        else:
+            _check_f32_gpu(lv, "lattice_values", 3)
+        _require(lv.is_contiguous(), "lattice_values must be contiguous (a slot is loaded at a time)")
         _require(lv.shape[2] == self.nr_feat, f"lattice_values should be nr_levels x capacity x {self.nr_feat}")
         levels = lv.shape[0]
         shift = fp.m_random_shift_per_level
@@ -288,10 +318,11 @@ class EncodingWrapper:
         n = pos.shape[0]
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
         out = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
+        entry = lib().penc_forward_half if lv.dtype == torch.float16 else lib().penc_forward
         with torch.cuda.device(pos.device):
-            _check(lib().penc_forward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
-                                      _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(out),
-                                      int(fp.m_concat_points), fp.m_points_scaling, _stream()), "forward")
+            _check(entry(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                         _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(out),
+                         int(fp.m_concat_points), fp.m_points_scaling, _stream()), "forward")
         return out
 
     def backward(self, inp, grad_sliced_values_monolithic):
@@ -307,7 +338,8 @@ class EncodingWrapper:
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
         grad = grad_sliced_values_monolithic
         self._check_grad(grad, levels, extra, n, allow_rows=True)
-        lv_grad = torch.empty_like(lv) if inp.m_require_lattice_values_grad else None
+        half = lv.dtype == torch.float16  # the gradient w.r.t. the table is fp32 either way
+        lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device) if inp.m_require_lattice_values_grad else None
         pos_grad = torch.empty_like(pos) if inp.m_require_positions_grad else None
         if lv_grad is None and pos_grad is None:
             return None, None
@@ -316,13 +348,19 @@ class EncodingWrapper:
                 copy_bytes = 4 * self.nr_feat * levels * n + 512 if pos_grad is not None else 0
                 ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None,
                                        fixed_bytes=copy_bytes, required_bytes=copy_bytes, nr_feat=self.nr_feat)
-                _check(lib().penc_backward_rowmajor(
+                _check((lib().penc_backward_half if half else lib().penc_backward_rowmajor)(
                     self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
                     _ptr(win), _ptr(grad), grad.stride(2), _ptr(lv_grad), _ptr(pos_grad), _ptr(ws),
                     0 if ws is None else ws.numel(), _stream()), "backward")
                 return lv_grad, pos_grad
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None,
                                    nr_feat=self.nr_feat)
+            if half:
+                _check(lib().penc_backward_half(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                                                _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(grad), 0, _ptr(lv_grad),
+                                                _ptr(pos_grad), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
+                       "backward")
+                return lv_grad, pos_grad
             _check(lib().penc_backward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
                                        _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(grad), _ptr(lv_grad),
                                        _ptr(pos_grad), _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
@@ -341,10 +379,17 @@ class EncodingWrapper:
         _check_f32_gpu(double_positions_grad, "double_positions_grad", 2)
         _require(double_positions_grad.shape == pos.shape, "double_positions_grad should be nr_positions x pos_dim")
         dpos = double_positions_grad.contiguous()
-        lv_grad = torch.empty_like(lv)
+        lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device)
         ggs = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
         with torch.cuda.device(pos.device):
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, nr_feat=self.nr_feat)
+            if lv.dtype == torch.float16:
+                _check(lib().penc_double_backward_from_positions_half(
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    _ptr(win), _ptr(dpos), _ptr(grad), 0 if grad.is_contiguous() else grad.stride(2), _ptr(lv_grad), _ptr(ggs),
+                    int(fp.m_concat_points), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
+                    "double_backward_from_positions")
+                return lv_grad, ggs
             if not grad.is_contiguous():
                 _check(lib().penc_double_backward_from_positions_rowmajor(
                     self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),

@@ -14,10 +14,12 @@
 //       bins, direct atomics) is described in penc_scatter.hpp.
 //   A level whose anneal-window weight is exactly 0 contributes exactly 0 everywhere (for finite
 //   table values), so such levels skip the table traffic and only store their zeros.
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "../../include/penc.h"
 #include "penc_lattice.hpp"
@@ -41,21 +43,35 @@ __device__ __forceinline__ fvec<D> load_point(const float* __restrict__ position
     return pos;
 }
 
-// The D+1 table entries of a simplex (F features each: an 8-byte or one or two 16-byte loads per vertex), fetched
-// back to back so that all loads are in flight together.  f[k][r] is feature k of vertex r.
+// The D+1 table entries of a simplex (F features each: one load of F elements per vertex, two of 16
+// bytes for eight floats), fetched back to back so that all loads are in flight together.
+// f[k][r] is feature k of vertex r.  T is the table's element type: float, or __half for a table
+// kept in half precision (the values are widened exactly; all arithmetic stays fp32).
 template <int D, int F>
 struct Vertices {
     fvec<D + 1> f[F];
 };
-template <int D, int F>
-__device__ __forceinline__ Vertices<D, F> load_vertices(const float* __restrict__ level_table, uvec<D + 1> h,
+template <int D, int F, typename T>
+__device__ __forceinline__ Vertices<D, F> load_vertices(const T* __restrict__ level_table, uvec<D + 1> h,
                                                         uint32_t capacity, uint32_t cap_mask) {
     static_assert(F == 2 || F == 4 || F == 8, "two, four or eight features per level");
     Vertices<D, F> v;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
         const size_t slot = to_slot(h[r], capacity, cap_mask);
-        if constexpr (F == 2) {
+        if constexpr (sizeof(T) == 2) {
+            // F halves in one load of 4, 8 or 16 bytes
+            using Packed = typename std::conditional<F == 2, uint32_t, typename std::conditional<F == 4, uint2, uint4>::type>::type;
+            const Packed raw = *reinterpret_cast<const Packed*>(level_table + F * slot);
+            uint32_t words[F / 2];
+            __builtin_memcpy(words, &raw, sizeof(raw));
+            static_for<F / 2>(PENC_BODY(q) {
+                PENC_INDEX(q);
+                const float2 x = __half22float2(__builtin_bit_cast(__half2, words[q]));
+                v.f[2 * q + 0][r] = x.x;
+                v.f[2 * q + 1][r] = x.y;
+            });
+        } else if constexpr (F == 2) {
             const float2 x = *reinterpret_cast<const float2*>(level_table + 2 * slot);
             v.f[0][r] = x.x;
             v.f[1][r] = x.y;
@@ -84,10 +100,10 @@ __device__ __forceinline__ Vertices<D, F> load_vertices(const float* __restrict_
 // (compute-bound) and a fine (gather-bound) level, which takes the fine level's slice out of L2
 // (30% slower).
 
-template <int D, int F>
+template <int D, int F, typename T>
 __global__ void __launch_bounds__(kBlock)
 forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
-               const float* __restrict__ positions, const float* __restrict__ table,
+               const float* __restrict__ positions, const T* __restrict__ table,
                const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                const float* __restrict__ window, float* __restrict__ sliced, float points_scaling) {
     const int n = blockIdx.x * kBlock + threadIdx.x;
@@ -118,7 +134,7 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
     fvec<D + 1> sorted;
     sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, s.delta, s.hash0, sorted, h);
     const fvec<D + 1> w = barycentric_of_sorted<D>(sorted);
-    const Vertices<D, F> v = load_vertices<D, F>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+    const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
     fvec<F> acc = 0.0f;
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
@@ -267,10 +283,10 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
 // the whole chip on the same few levels at a time (their table slices stay in L2) and give the
 // launch many more, shorter waves than one thread per point walking all levels.  (Doing this
 // kernel's rank permutations through LDS, as the forward does, was measured: no gain.)
-template <int D, int F>
+template <int D, int F, typename T>
 __global__ void __launch_bounds__(kBlock)
 backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t capacity, uint32_t cap_mask,
-                    const float* __restrict__ positions, const float* __restrict__ table,
+                    const float* __restrict__ positions, const T* __restrict__ table,
                     const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                     const float* __restrict__ window, const float* __restrict__ grad_sliced,
                     float* __restrict__ out) {
@@ -290,7 +306,7 @@ backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t c
         const float* sf = scale_factor + level * D;
         const Located<D> s = locate<D>(pos, random_shift + level * D, sf);
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
-        const Vertices<D, F> v = load_vertices<D, F>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+        const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
         const float* gp = grad_sliced + (static_cast<size_t>(level) * F) * n_points + n;
         fvec<D + 1> dB = (v.f[0] * w_level) * gp[0];  // :688-689, feature by feature
         static_for<F - 1>(PENC_BODY(kk) {
@@ -325,10 +341,10 @@ reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size
 // was measured 7-13% slower than the two: the gathering half wants small workgroups, the scattering
 // half large groups of points with the levels interleaved.)
 
-template <int D, int F>
+template <int D, int F, typename T>
 __global__ void __launch_bounds__(kBlock)
 grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
-                 const float* __restrict__ positions, const float* __restrict__ table,
+                 const float* __restrict__ positions, const T* __restrict__ table,
                  const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                  const float* __restrict__ window, const float* __restrict__ double_pos_grad,
                  float* __restrict__ grad_grad_sliced) {
@@ -351,7 +367,7 @@ grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mas
     fvec<D + 1> sorted;
     sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, pos_grad_grad_to_elevated<D>(load_point<D>(double_pos_grad, n), sf),
                         s.hash0, sorted, h);
-    const Vertices<D, F> v = load_vertices<D, F>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+    const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
     // dB[r] * w_level, then times the vertex value (:1484-1485)
     const fvec<D + 1> wr = sorted_elevated_grad_to_bary<D>(sorted) * w_level;
     fvec<F> gg = 0.0f;
@@ -469,8 +485,16 @@ inline int check_geometry(int pos_dim, int nr_feat, int64_t n, int levels, int c
 }
 
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
-// the table is gathered with 8-byte loads for two features and 16-byte loads for four or eight
-inline bool table_aligned(const void* p, int nr_feat) { return (reinterpret_cast<uintptr_t>(p) & (nr_feat >= 4 ? 15u : 7u)) == 0; }
+// The table as the gathering kernels see it: fp32, or half precision (the *_half entry points).
+struct TableRef {
+    const void* values;
+    bool half;
+};
+// a slot is gathered with one load (two of 16 bytes for eight floats): 4 to 16 bytes
+inline bool table_aligned(const TableRef& t, int nr_feat) {
+    const unsigned slot_bytes = static_cast<unsigned>(nr_feat) * (t.half ? 2u : 4u);
+    return (reinterpret_cast<uintptr_t>(t.values) & ((slot_bytes < 16u ? slot_bytes : 16u) - 1u)) == 0;
+}
 
 // Clears the table gradient with a fill kernel (float2 granularity: the array is only guaranteed
 // 8-byte alignment).  A kernel rather than hipMemsetAsync so that callers may capture the call in
@@ -606,6 +630,16 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
         PENC_DISPATCH_D(D_, __VA_ARGS__)                                \
     }
 
+// The same with the table's element type (float or __half) as TT.
+#define PENC_DISPATCH_DFT(D_, F_, HALF_, ...)                           \
+    if (HALF_) {                                                        \
+        using TT = __half;                                              \
+        PENC_DISPATCH_DF(D_, F_, __VA_ARGS__)                           \
+    } else {                                                            \
+        using TT = float;                                               \
+        PENC_DISPATCH_DF(D_, F_, __VA_ARGS__)                           \
+    }
+
 inline unsigned tiles(int64_t n) { return static_cast<unsigned>((n + kBlock - 1) / kBlock); }
 
 // Device address of this GPU's copy of `scratch`, looked up on the first call with that GPU
@@ -702,7 +736,7 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
 // levels in groups of pos_levels_per_group() when the workspace can hold the partial sums, else one
 // thread per point walks all levels.
 static int positions_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
-                              const float* lattice_values, const float* scale_factor, const float* random_shift,
+                              const TableRef& table, const float* scale_factor, const float* random_shift,
                               const float* anneal_window, const float* grad_level_major, float* positions_grad,
                               void* workspace, size_t workspace_bytes, hipStream_t st) {
     const int n = static_cast<int>(nr_positions);
@@ -718,10 +752,11 @@ static int positions_backward(int pos_dim, int nr_feat, int64_t nr_positions, in
         groups = want_groups;
         partial = reinterpret_cast<float*>(ws);
     }
-    PENC_DISPATCH_DF(pos_dim, nr_feat, hipLaunchKernelGGL((backward_pos_kernel<DD, FF>), dim3(tiles(nr_positions), groups),
-                                                         dim3(kBlock), 0, st, n, nr_levels, per_group, cap, mask, positions,
-                                                         lattice_values, scale_factor, random_shift, anneal_window,
-                                                         grad_level_major, partial));
+    PENC_DISPATCH_DFT(pos_dim, nr_feat, table.half,
+                      hipLaunchKernelGGL((backward_pos_kernel<DD, FF, TT>), dim3(tiles(nr_positions), groups), dim3(kBlock), 0,
+                                         st, n, nr_levels, per_group, cap, mask, positions,
+                                         static_cast<const TT*>(table.values), scale_factor, random_shift, anneal_window,
+                                         grad_level_major, partial));
     if (int rc = check_launch()) return rc;
     if (groups > 1) {
         const size_t want = (n_values + kBlock * 4 - 1) / (kBlock * 4);
@@ -743,7 +778,7 @@ static int transpose_rows(const float* src, int64_t src_row_stride, float* dst, 
 // penc_backward and penc_backward_static: argument checks, then the table gradient (clear, scatter,
 // reduce) and the position gradient on the same stream.
 static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                         const float* positions, const float* lattice_values, const float* scale_factor,
+                         const float* positions, const TableRef& table, const float* scale_factor,
                          const float* random_shift, const float* anneal_window,
                          const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                          void* workspace, size_t workspace_bytes, void* stream) {
@@ -751,8 +786,8 @@ static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
     if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_sliced_values)
         return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
-    if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
-    if ((lattice_values && !table_aligned(lattice_values, nr_feat)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    if (positions_grad && !table.values) return PENC_ERR_NULL_POINTER;
+    if ((table.values && !table_aligned(table, nr_feat)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (lattice_values_grad)
         if (int rc = table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
@@ -760,9 +795,28 @@ static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                                     workspace_bytes, st))
             return rc;
     if (positions_grad)
-        return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+        return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor,
                                   random_shift, anneal_window, grad_sliced_values, positions_grad, workspace, workspace_bytes, st);
     return PENC_OK;
+}
+
+static int forward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                        const float* positions, const TableRef& table, const float* scale_factor,
+                        const float* random_shift, const float* anneal_window, float* sliced_values,
+                        int concat_points, float points_scaling, void* stream) {
+    const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
+    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
+    if (!positions || !table.values || !scale_factor || !random_shift || !anneal_window || !sliced_values)
+        return PENC_ERR_NULL_POINTER;
+    if (!table_aligned(table, nr_feat)) return PENC_ERR_MISALIGNED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid(tiles(nr_positions), nr_levels + extra);
+    PENC_DISPATCH_DFT(pos_dim, nr_feat, table.half,
+                      hipLaunchKernelGGL((forward_kernel<DD, FF, TT>), grid, dim3(kBlock), 0, st,
+                                         static_cast<int>(nr_positions), nr_levels, static_cast<uint32_t>(capacity),
+                                         mask_of(capacity), positions, static_cast<const TT*>(table.values), scale_factor,
+                                         random_shift, anneal_window, sliced_values, points_scaling));
+    return check_launch();
 }
 
 extern "C" {
@@ -774,7 +828,7 @@ const char* penc_status_string(int status) {
         case PENC_ERR_BAD_SIZE: return "nr_positions, nr_levels and capacity must be positive and every array must stay below 2^31 elements";
         case PENC_ERR_UNSUPPORTED_POS_DIM: return "pos_dim must be 2,3,4,5,6,7 or 8";
         case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2, 4 or 8";
-        case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to 8 bytes for two features per level and to 16 for four or eight, lattice_values_grad and gradient rows to 8 bytes";
+        case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to one slot (at most 16 bytes), lattice_values_grad and gradient rows to 8 bytes";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
         case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major copy of the upstream gradient (penc_backward_rowmajor_workspace_bytes)";
         case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
@@ -828,19 +882,16 @@ int penc_forward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, 
                  const float* positions, const float* lattice_values, const float* scale_factor,
                  const float* random_shift, const float* anneal_window, float* sliced_values,
                  int concat_points, float points_scaling, void* stream) {
-    const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
-    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
-    if (!positions || !lattice_values || !scale_factor || !random_shift || !anneal_window || !sliced_values)
-        return PENC_ERR_NULL_POINTER;
-    if (!table_aligned(lattice_values, nr_feat)) return PENC_ERR_MISALIGNED;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 grid(tiles(nr_positions), nr_levels + extra);
-    PENC_DISPATCH_DF(pos_dim, nr_feat, hipLaunchKernelGGL((forward_kernel<DD, FF>), grid, dim3(kBlock), 0, st,
-                                                         static_cast<int>(nr_positions), nr_levels,
-                                                         static_cast<uint32_t>(capacity), mask_of(capacity), positions,
-                                                         lattice_values, scale_factor, random_shift, anneal_window,
-                                                         sliced_values, points_scaling));
-    return check_launch();
+    return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+                        scale_factor, random_shift, anneal_window, sliced_values, concat_points, points_scaling, stream);
+}
+
+int penc_forward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                      const float* positions, const void* lattice_values_half, const float* scale_factor,
+                      const float* random_shift, const float* anneal_window, float* sliced_values,
+                      int concat_points, float points_scaling, void* stream) {
+    return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values_half, true},
+                        scale_factor, random_shift, anneal_window, sliced_values, concat_points, points_scaling, stream);
 }
 
 int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
@@ -848,9 +899,9 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* random_shift, const float* anneal_window,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                   void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
-                         random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad, workspace,
-                         workspace_bytes, stream);
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+                         scale_factor, random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad,
+                         workspace, workspace_bytes, stream);
 }
 
 size_t penc_static_scratch_bytes(void) { return PENC_STATIC_SCRATCH_BYTES; }
@@ -868,8 +919,8 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
         return PENC_ERR_SCRATCH_TOO_SMALL;
     void* ws = static_scratch_of_current_device();
     if (ws == nullptr) return PENC_ERR_LAUNCH;
-    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
-                         random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad, ws,
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+                         scale_factor, random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad, ws,
                          PENC_STATIC_SCRATCH_BYTES, stream);
 }
 
@@ -895,17 +946,17 @@ size_t penc_backward_rowmajor_workspace_bytes(int pos_dim, int nr_feat, int64_t 
     return 512 + copy + (scratch > partial ? scratch : partial);
 }
 
-int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                           const float* positions, const float* lattice_values, const float* scale_factor,
-                           const float* random_shift, const float* anneal_window, const float* grad_rows,
-                           int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
-                           void* workspace, size_t workspace_bytes, void* stream) {
+static int backward_rowmajor_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                  const float* positions, const TableRef& table, const float* scale_factor,
+                                  const float* random_shift, const float* anneal_window, const float* grad_rows,
+                                  int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
     if (!positions || !scale_factor || !random_shift || !anneal_window) return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
-    if (positions_grad && !lattice_values) return PENC_ERR_NULL_POINTER;
+    if (positions_grad && !table.values) return PENC_ERR_NULL_POINTER;
     if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
-    if ((lattice_values && !table_aligned(lattice_values, nr_feat)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    if ((table.values && !table_aligned(table, nr_feat)) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (!positions_grad)
         return table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
@@ -932,8 +983,32 @@ int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int n
         if (cols > 255) return PENC_ERR_BAD_SIZE;
         if (int rc = transpose_rows(grad_rows, grad_row_stride, level_major, nr_positions, cols, st)) return rc;
     }
-    return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values, scale_factor,
+    return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor,
                               random_shift, anneal_window, level_major, positions_grad, rest, rest_bytes, st);
+}
+
+int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                           const float* positions, const float* lattice_values, const float* scale_factor,
+                           const float* random_shift, const float* anneal_window, const float* grad_rows,
+                           int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+    return backward_rowmajor_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+                                  scale_factor, random_shift, anneal_window, grad_rows, grad_row_stride, lattice_values_grad,
+                                  positions_grad, workspace, workspace_bytes, stream);
+}
+
+int penc_backward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                       const float* positions, const void* lattice_values_half, const float* scale_factor,
+                       const float* random_shift, const float* anneal_window, const float* grad,
+                       int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+    const TableRef table{lattice_values_half, true};
+    if (grad_row_stride != 0)
+        return backward_rowmajor_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor,
+                                      random_shift, anneal_window, grad, grad_row_stride, lattice_values_grad, positions_grad,
+                                      workspace, workspace_bytes, stream);
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor, random_shift,
+                         anneal_window, grad, lattice_values_grad, positions_grad, workspace, workspace_bytes, stream);
 }
 
 int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
@@ -947,26 +1022,26 @@ int penc_backward_table_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions,
 }
 
 static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                                const float* positions, const float* lattice_values, const float* scale_factor,
+                                const float* positions, const TableRef& table, const float* scale_factor,
                                 const float* random_shift, const float* anneal_window,
                                 const float* double_positions_grad, const float* grad, int64_t grad_row_stride,
                                 float* lattice_values_grad, float* grad_grad_sliced_values, int concat_points,
                                 void* workspace, size_t workspace_bytes, void* stream) {
     const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
-    if (!positions || !lattice_values || !scale_factor || !random_shift || !anneal_window ||
+    if (!positions || !table.values || !scale_factor || !random_shift || !anneal_window ||
         !double_positions_grad || !grad)
         return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !grad_grad_sliced_values) return PENC_ERR_NULL_POINTER;
-    if (!table_aligned(lattice_values, nr_feat) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
+    if (!table_aligned(table, nr_feat) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (grad_grad_sliced_values) {
         const dim3 grid(tiles(nr_positions), nr_levels + extra);
-        PENC_DISPATCH_DF(pos_dim, nr_feat, hipLaunchKernelGGL((grad_grad_kernel<DD, FF>), grid, dim3(kBlock), 0, st,
-                                                             static_cast<int>(nr_positions), nr_levels,
-                                                             static_cast<uint32_t>(capacity), mask_of(capacity), positions,
-                                                             lattice_values, scale_factor, random_shift, anneal_window,
-                                                             double_positions_grad, grad_grad_sliced_values));
+        PENC_DISPATCH_DFT(pos_dim, nr_feat, table.half,
+                          hipLaunchKernelGGL((grad_grad_kernel<DD, FF, TT>), grid, dim3(kBlock), 0, st,
+                                             static_cast<int>(nr_positions), nr_levels, static_cast<uint32_t>(capacity),
+                                             mask_of(capacity), positions, static_cast<const TT*>(table.values), scale_factor,
+                                             random_shift, anneal_window, double_positions_grad, grad_grad_sliced_values));
         if (int rc = check_launch()) return rc;
     }
     if (!lattice_values_grad) return PENC_OK;
@@ -983,7 +1058,7 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
                                         const float* grad_sliced_values, float* lattice_values_grad,
                                         float* grad_grad_sliced_values, int concat_points, void* workspace,
                                         size_t workspace_bytes, void* stream) {
-    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values,
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
                                 scale_factor, random_shift, anneal_window, double_positions_grad, grad_sliced_values, 0,
                                 lattice_values_grad, grad_grad_sliced_values, concat_points, workspace, workspace_bytes,
                                 stream);
@@ -999,10 +1074,25 @@ int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64
                                                  void* stream) {
     if (nr_levels > 0 && nr_positions > 0)
         if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
-    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, lattice_values,
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
                                 scale_factor, random_shift, anneal_window, double_positions_grad, grad_rows,
                                 grad_row_stride, lattice_values_grad, grad_grad_sliced_values, concat_points, workspace,
                                 workspace_bytes, stream);
+}
+
+int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                             const float* positions, const void* lattice_values_half,
+                                             const float* scale_factor, const float* random_shift,
+                                             const float* anneal_window, const float* double_positions_grad,
+                                             const float* grad, int64_t grad_row_stride, float* lattice_values_grad,
+                                             float* grad_grad_sliced_values, int concat_points, void* workspace,
+                                             size_t workspace_bytes, void* stream) {
+    if (grad_row_stride != 0 && nr_levels > 0 && nr_positions > 0)
+        if (int rc = check_rows(grad, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions,
+                                TableRef{lattice_values_half, true}, scale_factor, random_shift, anneal_window,
+                                double_positions_grad, grad, grad_row_stride, lattice_values_grad, grad_grad_sliced_values,
+                                concat_points, workspace, workspace_bytes, stream);
 }
 
 int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream) {

@@ -364,3 +364,43 @@ def test_module_with_more_features_per_level(feat):
     r = orc.double_backward(p, t, sf, sh, w, q.cpu().numpy(), g, want_abs=True)
     err = np.abs(m.lattice_values.grad.cpu().numpy() - r["grad64"])
     assert np.all(err <= 1e-4 * r["abs64"] + 1e-30)
+
+
+def test_module_gathers_from_a_half_precision_copy():
+    """PermutoEncoding(..., lattice_half_precision=True): the kernels gather from a float16 copy of the
+    fp32 parameter; the output is that of the rounded table, gradients reach the fp32 parameter in fp32
+    (first and second order), and the copy follows in-place updates of the parameter."""
+    import permutohedral_encoding_amd as pe
+    torch.manual_seed(3)
+    levels, n = 5, 2000
+    m = pe.PermutoEncoding(3, 1 << 12, levels, 2, np.geomspace(1.0, 1e-2, levels), lattice_half_precision=True)
+    with torch.no_grad():
+        m.lattice_values.uniform_(-1, 1)
+    pos = torch.rand(n, 3, device="cuda", requires_grad=True)
+    out = m(pos)
+    p, t, sf, sh = oracle_args(m, pos)
+    rounded = t.astype(np.float16).astype(np.float32)
+    assert not np.array_equal(rounded, t)
+    w = np.ones(levels, np.float32)
+    want = orc.forward(p, rounded, sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
+    assert np.array_equal(out.detach().cpu().numpy(), want)
+    up = torch.randn(n, 2 * levels, device="cuda")
+    grad_pos, = torch.autograd.grad(out, pos, up, create_graph=True)
+    g = up.cpu().numpy().reshape(n, levels, 2).transpose(1, 2, 0).copy()
+    wp = orc.backward_pos(p, rounded, sf, sh, w, g)
+    assert np.all(np.abs(grad_pos.detach().cpu().numpy() - wp["grad64"]) <= 1e-6 * wp["abs64"] + 1e-30)
+    q = torch.randn(n, 3, device="cuda")
+    (grad_pos * q).sum().backward()
+    assert m.lattice_values.grad.dtype == torch.float32 and m.lattice_values.dtype == torch.float32
+    r = orc.double_backward(p, rounded, sf, sh, w, q.cpu().numpy(), g, want_abs=True)
+    assert np.all(np.abs(m.lattice_values.grad.cpu().numpy() - r["grad64"]) <= 1e-4 * r["abs64"] + 1e-30)
+    # an optimizer step modifies the parameter in place: the next forward reads a fresh copy
+    with torch.no_grad():
+        m.lattice_values.mul_(0.5)
+    out2 = m(pos.detach())
+    want2 = orc.forward(p, (0.5 * t).astype(np.float16).astype(np.float32), sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
+    assert np.array_equal(out2.detach().cpu().numpy(), want2)
+    # pickling keeps the switch
+    import pickle
+    m2 = pickle.loads(pickle.dumps(m))
+    assert m2.lattice_half_precision and torch.equal(m2(pos.detach()), out2)

@@ -232,6 +232,44 @@ def test_more_features_at_benchmark_size_with_rows_and_concat_points(feat, n):
     check_grad_grad(ggs.cpu().numpy(), want)
 
 
+# ----------------------------------------------------------------------------- table in half precision
+
+@pytest.mark.parametrize("feat", [2, 4, 8])
+@pytest.mark.parametrize("d", [2, 3, 4, 8])
+def test_half_precision_table_equals_the_widened_table(d, feat):
+    """A float16 table through the *_half entry points: the kernels widen on load and compute in fp32, so
+    every result is that of the fp32 path on the widened table: forward and grad-of-grad bit-equal to the
+    oracle run on it, position gradient within its bound, table gradients (which never read the table)
+    fp32 as before.  Level-major and row-major upstream gradients."""
+    from permutohedral_encoding_amd import _native
+    cap = (1 << 12) if d != 3 else 5001  # odd capacity: slots of 2F bytes at odd offsets
+    n, levels = 5000, 4
+    p = random_problem(d, n, levels, cap, seed=130 + d + feat, sigma_range=(1.0, 1e-3), nr_feat=feat)
+    half = p["table"].astype(np.float16)
+    p["table"] = half.astype(np.float32)
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
+    inp = gpu_input(p)
+    inp.m_lattice_values = to_gpu(half)
+    out = enc.forward(inp).cpu().numpy()
+    assert np.array_equal(out, orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"]))
+    rows = to_gpu(np.ascontiguousarray(p["grad"].transpose(2, 0, 1).reshape(n, levels * feat)))
+    view = rows.reshape(n, levels, feat).permute(1, 2, 0)
+    assert _native.is_row_major_view(view)
+    want_t = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    want_p = orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"])
+    want_d = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    for grad in (to_gpu(p["grad"]), view):
+        tg, pg = enc.backward(inp, grad)
+        assert tg.dtype == torch.float32 and tg.shape == (levels, cap, feat)
+        assert_sum_close(tg.cpu().numpy(), want_t["grad64"], want_t["abs64"], SUM_RTOL, "table gradient, half table")
+        check_pos_grad(pg.cpu().numpy(), want_p)
+        tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), grad)
+        assert tg2.dtype == torch.float32
+        assert_sum_close(tg2.cpu().numpy(), want_d["grad64"], want_d["abs64"], SUM_RTOL, "second-order table gradient, half table")
+        check_grad_grad(ggs.cpu().numpy(), want_d)
+
+
 # ----------------------------------------------------------------------------- edge cases
 
 @pytest.mark.parametrize("n", [1, 63, 64, 65, 255, 256, 257, 4095, 4097, 10001])
