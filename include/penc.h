@@ -212,6 +212,17 @@ int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t n
                                              float* grad_grad_sliced_values, int concat_points, void* workspace,
                                              size_t workspace_bytes, void* stream);
 
+/* One AdamW step (decoupled weight decay, no amsgrad) on n fp32 values in a single kernel, with the
+ * formulas and the order of operations of torch.optim.AdamW; `step` counts from 1.  With
+ * skip_zero_gradients an entry whose gradient is exactly 0 keeps its value and both moments: on a
+ * hash table most slots receive no gradient in a step, and the update then reads the gradient and
+ * touches the rest only where something arrived.
+ * No counterpart in the reference library; its training script steps the whole table with
+ * torch.optim.AdamW (examples/performance.py:99-101, 161). */
+int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* exp_avg_sq, int64_t n, double lr,
+                    double beta1, double beta2, double eps, double weight_decay, int64_t step, int skip_zero_gradients,
+                    void* stream);
+
 /* dst[c][r] = src[r][c] for a dense row-major rows x cols matrix with cols <= 255 (2 * levels):
  * turns the row-major upstream gradient (N, 2(L+E)) into the grad_sliced_values layout
  * [L+E][2][N] at streaming speed.

@@ -64,6 +64,9 @@ _SIGNATURES = {
                                                                 _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
                                                                 _c_f32p, ctypes.c_int, ctypes.c_void_p,
                                                                 ctypes.c_size_t, ctypes.c_void_p]),
+    "penc_adamw_step": (ctypes.c_int, [_c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_double, ctypes.c_double,
+                                       ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_int64, ctypes.c_int,
+                                       ctypes.c_void_p]),
     "penc_transpose": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
                                           _c_f32p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,

@@ -381,6 +381,58 @@ grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mas
 }
 
 // ------------------------------------------------------------------------------------------
+// optimiser step on the table
+
+// One fused AdamW update (decoupled weight decay, no amsgrad) in the order torch.optim.AdamW applies
+// it: p *= 1 - lr*wd; m += (1-b1)(g - m); v = b2 v + (1-b2) g^2; p -= step_size * m / (sqrt(v)/c2 + eps).
+// With skip_zero an entry whose gradient is exactly 0 is left alone altogether (moments, decay and
+// value), which is how hash-grid tables are usually trained: most slots of a large table get no
+// gradient in a step.  Four values per thread where the arrays allow 16-byte accesses.
+struct AdamWStep {
+    float decay;        // 1 - lr * weight_decay
+    float one_minus_b1, b2, one_minus_b2;
+    float step_size;    // lr / (1 - b1^step)
+    float inv_c2;       // 1 / sqrt(1 - b2^step)
+    float eps;
+};
+__device__ __forceinline__ void adamw_update(const AdamWStep& a, bool skip_zero, float g, float& p, float& m, float& v) {
+    if (skip_zero && g == 0.0f) return;
+    p = p * a.decay;
+    m = m + a.one_minus_b1 * (g - m);
+    v = v * a.b2 + a.one_minus_b2 * (g * g);
+    p = p - a.step_size * (m / (__builtin_sqrtf(v) * a.inv_c2 + a.eps));
+}
+template <bool kVector>
+__global__ void __launch_bounds__(kBlock)
+adamw_step_kernel(float* __restrict__ params, const float* __restrict__ grads, float* __restrict__ exp_avg,
+                  float* __restrict__ exp_avg_sq, size_t n, AdamWStep a, int skip_zero) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    if constexpr (kVector) {
+        if (i * 4 >= n) return;
+        const float4 g = reinterpret_cast<const float4*>(grads)[i];
+        if (skip_zero && g.x == 0.0f && g.y == 0.0f && g.z == 0.0f && g.w == 0.0f) return;
+        float4 p = reinterpret_cast<float4*>(params)[i], m = reinterpret_cast<float4*>(exp_avg)[i],
+               v = reinterpret_cast<float4*>(exp_avg_sq)[i];
+        adamw_update(a, skip_zero, g.x, p.x, m.x, v.x);
+        adamw_update(a, skip_zero, g.y, p.y, m.y, v.y);
+        adamw_update(a, skip_zero, g.z, p.z, m.z, v.z);
+        adamw_update(a, skip_zero, g.w, p.w, m.w, v.w);
+        reinterpret_cast<float4*>(params)[i] = p;
+        reinterpret_cast<float4*>(exp_avg)[i] = m;
+        reinterpret_cast<float4*>(exp_avg_sq)[i] = v;
+    } else {
+        if (i >= n) return;
+        float p = params[i], m = exp_avg[i], v = exp_avg_sq[i];
+        const float g = grads[i];
+        if (skip_zero && g == 0.0f) return;
+        adamw_update(a, skip_zero, g, p, m, v);
+        params[i] = p;
+        exp_avg[i] = m;
+        exp_avg_sq[i] = v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // introspection
 
 // kViaLds selects which of the two equivalent device routines produce the slots and weights: the
@@ -1093,6 +1145,44 @@ int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t n
                                 TableRef{lattice_values_half, true}, scale_factor, random_shift, anneal_window,
                                 double_positions_grad, grad, grad_row_stride, lattice_values_grad, grad_grad_sliced_values,
                                 concat_points, workspace, workspace_bytes, stream);
+}
+
+int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* exp_avg_sq, int64_t n, double lr,
+                    double beta1, double beta2, double eps, double weight_decay, int64_t step, int skip_zero_gradients,
+                    void* stream) {
+    if (!params || !grads || !exp_avg || !exp_avg_sq) return PENC_ERR_NULL_POINTER;
+    if (n <= 0 || step <= 0) return PENC_ERR_BAD_SIZE;
+    // the scalars as torch.optim.AdamW forms them (in double), rounded once for the kernel
+    AdamWStep a;
+    a.decay = static_cast<float>(1.0 - lr * weight_decay);
+    a.one_minus_b1 = static_cast<float>(1.0 - beta1);
+    a.b2 = static_cast<float>(beta2);
+    a.one_minus_b2 = static_cast<float>(1.0 - beta2);
+    a.step_size = static_cast<float>(lr / (1.0 - __builtin_pow(beta1, static_cast<double>(step))));
+    a.inv_c2 = static_cast<float>(1.0 / __builtin_sqrt(1.0 - __builtin_pow(beta2, static_cast<double>(step))));
+    a.eps = static_cast<float>(eps);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uintptr_t all = reinterpret_cast<uintptr_t>(params) | reinterpret_cast<uintptr_t>(grads) |
+                          reinterpret_cast<uintptr_t>(exp_avg) | reinterpret_cast<uintptr_t>(exp_avg_sq);
+    const size_t count = static_cast<size_t>(n);
+    const size_t vector_part = (all & 15u) == 0 ? count / 4 * 4 : 0;
+    if (vector_part != 0) {
+        const size_t blocks = (vector_part / 4 + kBlock - 1) / kBlock;
+        if (blocks > 0x7FFFFFFFull) return PENC_ERR_BAD_SIZE;
+        hipLaunchKernelGGL(adamw_step_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, st, params, grads,
+                           exp_avg, exp_avg_sq, vector_part, a, skip_zero_gradients);
+        if (int rc = check_launch()) return rc;
+    }
+    if (vector_part != count) {
+        const size_t rest = count - vector_part;
+        const size_t blocks = (rest + kBlock - 1) / kBlock;
+        if (blocks > 0x7FFFFFFFull) return PENC_ERR_BAD_SIZE;
+        hipLaunchKernelGGL(adamw_step_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(kBlock), 0, st,
+                           params + vector_part, grads + vector_part, exp_avg + vector_part, exp_avg_sq + vector_part, rest, a,
+                           skip_zero_gradients);
+        if (int rc = check_launch()) return rc;
+    }
+    return PENC_OK;
 }
 
 int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream) {

@@ -14,7 +14,7 @@ Unlike the kernel benchmark (``bench.py``) these figures include everything a us
 pays: output allocation, the loss, the gradient layout change and the optimiser walking the whole
 table.
 
-    python -m permutohedral_encoding_amd.perf_sweep [--dims 2 3 4 5 6] [--points 524288] [--iters 300]
+    python -m permutohedral_encoding_amd.perf_sweep [--dims 2 3 4 5 6] [--points 524288] [--iters 300] [--fused-optimizer]
 """
 import argparse
 import json
@@ -39,10 +39,14 @@ def _timed(step, nr_points, iters, warmup):
     return float(np.mean(kept))
 
 
-def measure(pos_dim, nr_points, iters, warmup, levels=24, log2_capacity=18):
+def measure(pos_dim, nr_points, iters, warmup, levels=24, log2_capacity=18, fused_optimizer=False):
     torch.manual_seed(0)
     enc = PermutoEncoding(pos_dim, 1 << log2_capacity, levels, 2, np.geomspace(1.0, 1e-4, num=levels))
-    opt = torch.optim.AdamW(enc.parameters(), amsgrad=False, betas=(0.9, 0.99), eps=1e-15, weight_decay=0.0, lr=1e-3)
+    if fused_optimizer:  # the library's one-kernel AdamW instead of torch's (same update)
+        from .optim import AdamW
+        opt = AdamW(enc.parameters(), betas=(0.9, 0.99), eps=1e-15, weight_decay=0.0, lr=1e-3)
+    else:
+        opt = torch.optim.AdamW(enc.parameters(), amsgrad=False, betas=(0.9, 0.99), eps=1e-15, weight_decay=0.0, lr=1e-3)
     pts = torch.rand(nr_points, pos_dim, device="cuda") - 0.5
     pts_grad = pts.clone().requires_grad_(True)
 
@@ -71,6 +75,8 @@ def main():
     ap.add_argument("--points", type=int, default=1 << 19)
     ap.add_argument("--iters", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--fused-optimizer", action="store_true",
+                    help="step the table with permutohedral_encoding_amd.optim.AdamW instead of torch.optim.AdamW")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("perf_sweep: no GPU visible; the encoding has no CPU path")
@@ -78,7 +84,7 @@ def main():
     print("|---|---|---|---|")
     rows = []
     for d in args.dims:
-        r = measure(d, args.points, args.iters, args.warmup)
+        r = measure(d, args.points, args.iters, args.warmup, fused_optimizer=args.fused_optimizer)
         rows.append(r)
         print(f"| {d} | {r['inference']:.3g} | {r['train_table']:.3g} | {r['train_table_pos']:.3g} |", flush=True)
     print(json.dumps(rows))

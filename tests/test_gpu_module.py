@@ -404,3 +404,72 @@ def test_module_gathers_from_a_half_precision_copy():
     import pickle
     m2 = pickle.loads(pickle.dumps(m))
     assert m2.lattice_half_precision and torch.equal(m2(pos.detach()), out2)
+
+
+@pytest.mark.parametrize("n", [4096, 4099, 3])
+def test_fused_adamw_follows_torch_adamw(n):
+    """penc_adamw_step through permutohedral_encoding_amd.optim.AdamW against torch.optim.AdamW on the same
+    parameter and gradients, several steps, with weight decay; sizes that do and do not split into
+    16-byte accesses."""
+    from permutohedral_encoding_amd.optim import AdamW
+    torch.manual_seed(n)
+    start = torch.randn(n, device="cuda")
+    a = torch.nn.Parameter(start.clone())
+    b = torch.nn.Parameter(start.clone())
+    kw = dict(lr=3e-3, betas=(0.9, 0.99), eps=1e-8, weight_decay=0.05)
+    ours, theirs = AdamW([a], **kw), torch.optim.AdamW([b], **kw)
+    for step in range(6):
+        g = torch.randn(n, device="cuda") * (10.0 ** (step - 3))
+        a.grad, b.grad = g.clone(), g.clone()
+        version = a._version
+        ours.step()
+        theirs.step()
+        assert a._version > version  # in-place change recorded
+        assert torch.allclose(a, b, rtol=2e-6, atol=1e-7), (step, (a - b).abs().max().item())
+    sa, sb = ours.state[a], theirs.state[b]
+    # the moments are sums with cancellation: a few units in the last place of their largest terms
+    for key in ("exp_avg", "exp_avg_sq"):
+        assert torch.allclose(sa[key], sb[key], rtol=2e-6, atol=2e-6 * sb[key].abs().max().item()), key
+
+
+def test_fused_adamw_leaves_entries_without_gradient_alone():
+    """skip_zero_gradients: an entry with a zero gradient keeps its value and its moments (no decay of
+    either, no weight decay); the others are updated as by torch.optim.AdamW with the same step count."""
+    from permutohedral_encoding_amd.optim import AdamW
+    torch.manual_seed(5)
+    n = 10007
+    start = torch.randn(n, device="cuda")
+    a = torch.nn.Parameter(start.clone())
+    b = torch.nn.Parameter(start.clone())
+    kw = dict(lr=1e-2, betas=(0.9, 0.99), eps=1e-15, weight_decay=0.01)
+    ours, theirs = AdamW([a], skip_zero_gradients=True, **kw), torch.optim.AdamW([b], **kw)
+    touched = torch.rand(n, device="cuda") < 0.3
+    for step in range(4):
+        g = torch.randn(n, device="cuda") * touched
+        a.grad, b.grad = g.clone(), g.clone()
+        ours.step()
+        theirs.step()
+    assert torch.equal(a[~touched], start[~touched])
+    assert torch.all(ours.state[a]["exp_avg"][~touched] == 0) and torch.all(ours.state[a]["exp_avg_sq"][~touched] == 0)
+    assert torch.allclose(a[touched], b[touched], rtol=2e-6, atol=1e-7)
+
+
+def test_training_with_the_fused_optimizer_and_a_half_precision_table():
+    """A few steps of the reference's training protocol (loss ((pred-10)^2).mean(), zero_grad, backward,
+    step) with the fused optimizer on a module that gathers from a half-precision copy: the loss goes
+    down and the copy follows the optimizer's in-place updates."""
+    import permutohedral_encoding_amd as pe
+    from permutohedral_encoding_amd.optim import AdamW
+    torch.manual_seed(0)
+    m = pe.PermutoEncoding(3, 1 << 14, 8, 2, np.geomspace(1.0, 1e-2, 8), lattice_half_precision=True)
+    opt = AdamW(m.parameters(), lr=1e-1, betas=(0.9, 0.99), eps=1e-15, weight_decay=0.0, skip_zero_gradients=True)
+    pts = torch.rand(20000, 3, device="cuda") - 0.5
+    losses = []
+    for _ in range(8):
+        loss = ((m(pts) - 10) ** 2).mean()
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < 0.9 * losses[0], losses
+    assert all(later < earlier for earlier, later in zip(losses, losses[1:])), losses
