@@ -23,10 +23,11 @@
 //      private segment in every bin, so appending costs one LDS counter increment and one
 //      store); a second kernel (bin_reduce_kernel) reads each bin back coalesced, sums it in
 //      LDS (fp64), and adds the range into the gradient with coalesced read-modify-writes.  This
-//      turns the random scatter of the fine levels into streaming traffic.  Once a workgroup has
-//      seen that its cache does not hit at a level, it gives the cache's LDS to its wavefronts as
-//      staging space: the workgroup sorts the records of a tile by bin there, so that records of one
-//      bin leave in runs of consecutive addresses (whole cache lines) instead of one 12-byte store each.
+//      turns the random scatter of the fine levels into streaming traffic.  A workgroup whose
+//      look-up of the first tile's slots shows that the cache would not hit at its level never
+//      fills it: the cache's LDS becomes staging space in which the records of a tile are sorted by
+//      bin, so that records of one bin leave in runs of consecutive addresses (whole cache lines)
+//      instead of one 12-byte store each.
 //   3. Direct global atomics, with the two features of a slot in one instruction (lane pairs),
 //      for whatever is left: no workspace, capacity too large for binning, or a full bin.
 // The result never depends on a stage hitting: every stage falls through to the next.
