@@ -143,7 +143,10 @@ forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
             PENC_INDEX(k); acc[k] = acc[k] + v.f[k][r] * wr; });
     });
     static_for<F>(PENC_BODY(k) {
-        PENC_INDEX(k); out[static_cast<size_t>(k) * n_points] = acc[k]; });
+        PENC_INDEX(k);
+        // written once and not read here: the non-temporal hint keeps it from displacing the level's table slice
+        __builtin_nontemporal_store(acc[k], out + static_cast<size_t>(k) * n_points);
+    });
 }
 
 // ------------------------------------------------------------------------------------------
@@ -308,11 +311,12 @@ backward_pos_kernel(int n_points, int n_levels, int levels_per_group, uint32_t c
         const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
         const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
         const float* gp = grad_sliced + (static_cast<size_t>(level) * F) * n_points + n;
-        fvec<D + 1> dB = (v.f[0] * w_level) * gp[0];  // :688-689, feature by feature
+        // the upstream gradient is read once (non-temporal: it should not displace the table slices)
+        fvec<D + 1> dB = (v.f[0] * w_level) * __builtin_nontemporal_load(gp);  // :688-689, feature by feature
         static_for<F - 1>(PENC_BODY(kk) {
             PENC_INDEX(kk);
             constexpr int k = kk + 1;
-            dB += (v.f[k] * w_level) * gp[static_cast<size_t>(k) * n_points];
+            dB += (v.f[k] * w_level) * __builtin_nontemporal_load(gp + static_cast<size_t>(k) * n_points);
         });
         total += bary_grad_to_pos_grad<D>(s.rank, dB, sf);
     }
