@@ -677,6 +677,33 @@ def test_first_tile_misleads_the_scatter_about_the_level(d):
         _table_gradients_match(p, d, cap, what)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_table_gradients_on_mixed_point_distributions(seed):
+    """Clusters of random size and spread mixed with uniform points, random dimension, capacity, level
+    range and point count: levels land on either side of every threshold the scatter decides by
+    (distinct slots of the first tile, its hit rate, bins or no bins), some workgroups of a level on
+    one side and some on the other."""
+    rng = np.random.default_rng(1000 + seed)
+    d = int(rng.choice([2, 3, 4, 5]))
+    cap = int(rng.choice([1 << 12, 1 << 15, 1 << 18, 30011]))
+    n = int(rng.integers(3000, 40000))
+    levels = 6
+    fine = float(10.0 ** rng.uniform(-4, -1.5))
+    p = random_problem(d, n, levels, cap, seed=2000 + seed, sigma_range=(1.0, fine))
+    n_clusters = int(rng.integers(1, 40))
+    centres = rng.uniform(0, 1, (n_clusters, d))
+    spread = 10.0 ** rng.uniform(-6, -1, n_clusters)
+    member = rng.integers(0, n_clusters, n)
+    clustered = centres[member] + spread[member, None] * rng.standard_normal((n, d))
+    uniform = rng.uniform(0, 1, (n, d))
+    # runs of points alternate between the two kinds, so that the first tile of a group of points need not
+    # look like the rest of it
+    run = int(rng.choice([64, 512, 3000]))
+    pick = ((np.arange(n) // run) % 2 == 0) if rng.random() < 0.7 else (rng.random(n) < rng.uniform(0.1, 0.9))
+    p["pos"] = np.where(pick[:, None], clustered, uniform).astype(np.float32)
+    _table_gradients_match(p, d, cap, f"seed {seed}: D={d} cap={cap} n={n} clusters={n_clusters}")
+
+
 def test_records_crowd_one_bin():
     """Points chosen so that, at the finest level, at least three of their four vertices fall into the
     first of four slot ranges: the tile's records are all distinct (the workgroup streams them sorted
