@@ -394,9 +394,10 @@ __device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_gra
     });
 }
 
-// The same sort with every wave on its own (no barriers), for the dimensions whose D+1 vertices
-// take two chunks: the waves of a workgroup drift apart over their longer tiles, and waiting for
-// each other three times per chunk then costs more than the longer runs save (measured at D = 8).
+// The same sort with every wave on its own (no barriers), for the higher dimensions: their D+1
+// vertices take two chunks, the waves of a workgroup drift apart over their longer tiles, and
+// waiting for each other three times per chunk then costs more than the longer runs save
+// (measured: 5-7% slower at D = 6, 7, 8; D = 5, whose second chunk is a single vertex, still gains 4%).
 // The staging space is a 4 or 5 KiB slice per wave.  For stage_chunk(D) vertices per thread at a time, the wave
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
@@ -602,7 +603,7 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
                                                  uint32_t group, bool active, bool use_cache, int mode, uint32_t id_bits,
                                                  uvec<D + 1> slot, fvec<D + 1> a0, fvec<D + 1> a1) {
     if (mode == kModeStream) {
-        if constexpr (D + 1 <= State::kChunk) {
+        if constexpr (D <= 5) {  // measured: the workgroup-wide sort wins up to D = 5, the per-wave one from D = 6 on
             stream_tile<D>(c, level_grad, bins, group, active, slot, a0, a1);
         } else {
             stream_tile_wave<D>(c, level_grad, bins, group, active, slot, a0, a1);
