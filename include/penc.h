@@ -14,7 +14,7 @@
  *  - All arrays are fp32, densely packed, row-major (F = nr_feat, the features per level: 2, 4 or 8):
  *        positions            [N][D]
  *        lattice_values       [L][C][F]      (8-byte aligned for F = 2, 16-byte for F = 4 and 8;
- *                                            binary16 in the *_half entry points)
+ *                                            binary16 or bfloat16 in the *_half entry points)
  *        scale_factor         [L][D]         (from penc_scale_factors)
  *        random_shift         [L][D]
  *        anneal_window        [L]
@@ -56,6 +56,7 @@ extern "C" {
 #define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
 #define PENC_ERR_SCRATCH_TOO_SMALL 7    /* penc_backward_static: the problem does not fit the static scratch */
 #define PENC_ERR_WORKSPACE_TOO_SMALL 8  /* penc_backward_rowmajor with positions_grad: no room for the level-major copy */
+#define PENC_ERR_UNSUPPORTED_TABLE_FORMAT 9 /* the *_half entry points: table_format is neither PENC_TABLE_FP16 nor PENC_TABLE_BF16 */
 
 const char* penc_status_string(int status);
 
@@ -185,27 +186,30 @@ int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64
                                                  int concat_points, void* workspace, size_t workspace_bytes,
                                                  void* stream);
 
-/* The three gathering entry points for a table kept in half precision: lattice_values_half is
- * [L][C][F] of IEEE binary16 (aligned to one slot of 2F bytes).  The values are widened exactly
- * on load and all arithmetic stays fp32, so the results are those of the fp32 entry points on the
- * widened table; sliced values, both gradients and grad_grad_sliced_values are fp32 as before (the
- * table gradient never reads the table).  grad_row_stride selects the layout of the upstream
- * gradient: 0 for [L+E][F][N], otherwise rows of that many floats as in the *_rowmajor entry points
- * (with their workspace rules).
+/* The three gathering entry points for a table kept in 16 bits per value: lattice_values_half is
+ * [L][C][F] of IEEE binary16 (table_format PENC_TABLE_FP16) or of bfloat16 (PENC_TABLE_BF16),
+ * aligned to one slot of 2F bytes.  The values are widened exactly on load and all arithmetic
+ * stays fp32, so the results are those of the fp32 entry points on the widened table; sliced
+ * values, both gradients and grad_grad_sliced_values are fp32 as before (the table gradient never
+ * reads the table).  grad_row_stride selects the layout of the upstream gradient: 0 for
+ * [L+E][F][N], otherwise rows of that many floats as in the *_rowmajor entry points (with their
+ * workspace rules).
  * Replaces: nothing that runs in the reference; it carries the intent as a disabled switch
  * (LATTICE_HALF_PRECISION, kernels/permutohedral_encoding/EncodingGPU.cuh:12) beside the same
  * forward / backward / double_backward_from_positions (src/Encoding.cu:55-334). */
+#define PENC_TABLE_FP16 1
+#define PENC_TABLE_BF16 2
 int penc_forward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                      const float* positions, const void* lattice_values_half, const float* scale_factor,
-                      const float* random_shift, const float* anneal_window, float* sliced_values,
-                      int concat_points, float points_scaling, void* stream);
+                      const float* positions, const void* lattice_values_half, int table_format,
+                      const float* scale_factor, const float* random_shift, const float* anneal_window,
+                      float* sliced_values, int concat_points, float points_scaling, void* stream);
 int penc_backward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                       const float* positions, const void* lattice_values_half, const float* scale_factor,
-                       const float* random_shift, const float* anneal_window, const float* grad,
-                       int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                       const float* positions, const void* lattice_values_half, int table_format,
+                       const float* scale_factor, const float* random_shift, const float* anneal_window,
+                       const float* grad, int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
                        void* workspace, size_t workspace_bytes, void* stream);
 int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                                             const float* positions, const void* lattice_values_half,
+                                             const float* positions, const void* lattice_values_half, int table_format,
                                              const float* scale_factor, const float* random_shift,
                                              const float* anneal_window, const float* double_positions_grad,
                                              const float* grad, int64_t grad_row_stride, float* lattice_values_grad,

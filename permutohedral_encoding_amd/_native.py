@@ -54,13 +54,13 @@ _SIGNATURES = {
                                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int,
                                                            ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_forward_half": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
-                                         _c_f32p, ctypes.c_void_p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                         _c_f32p, ctypes.c_void_p, ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                          ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
     "penc_backward_half": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
-                                          _c_f32p, ctypes.c_void_p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
+                                          _c_f32p, ctypes.c_void_p, ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
                                           _c_f32p, _c_f32p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_double_backward_from_positions_half": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
-                                                                ctypes.c_int, _c_f32p, ctypes.c_void_p, _c_f32p, _c_f32p,
+                                                                ctypes.c_int, _c_f32p, ctypes.c_void_p, ctypes.c_int, _c_f32p, _c_f32p,
                                                                 _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p,
                                                                 _c_f32p, ctypes.c_int, ctypes.c_void_p,
                                                                 ctypes.c_size_t, ctypes.c_void_p]),
@@ -166,6 +166,9 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+TABLE_FORMATS = {torch.float16: 1, torch.bfloat16: 2}  # PENC_TABLE_FP16, PENC_TABLE_BF16 (include/penc.h)
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
@@ -261,18 +264,19 @@ class EncodingWrapper:
         return EncodingWrapper(pos_dim, nr_feat_per_level, fixed_params)
 
     # -- checks shared by the three calls (reference: src/Encoding.cu:38-45, 57-66, 119-125)
-    half_table = False  # set by the module: gather from a half-precision copy of the fp32 table
+    half_table = None  # set by the module: torch.float16 or torch.bfloat16 to gather from such a copy of the fp32 table
     _half_copy = None
     _half_copy_of = None
 
     def gather_table(self, lattice_values):
         """The tensor the gathering kernels read for ``lattice_values``: the tensor itself, or, with
-        ``half_table``, its float16 copy, made again whenever the tensor has been modified in place."""
-        if not self.half_table or lattice_values.dtype != torch.float32:
+        ``half_table``, its 16-bit copy, made again whenever the tensor has been modified in place."""
+        if self.half_table is None or lattice_values.dtype != torch.float32:
             return lattice_values
-        key = (lattice_values.data_ptr(), lattice_values._version, lattice_values.device, tuple(lattice_values.shape))
+        key = (lattice_values.data_ptr(), lattice_values._version, lattice_values.device, tuple(lattice_values.shape),
+               self.half_table)
         if self._half_copy_of != key:
-            self._half_copy = lattice_values.detach().to(torch.float16)
+            self._half_copy = lattice_values.detach().to(self.half_table)
             self._half_copy_of = key
         return self._half_copy
 
@@ -284,7 +288,7 @@ class EncodingWrapper:
         _require(pos.shape[1] == fp.m_pos_dim,
                  f"Pos dim for the lattice doesn't correspond with the position of the points. Lattice was initialized "
                  f"with {fp.m_pos_dim} and points have pos dim {pos.shape[1]}")
-        if isinstance(lv, torch.Tensor) and lv.dtype == torch.float16:  # a table kept in half precision: the *_half entry points
+        if isinstance(lv, torch.Tensor) and lv.dtype in TABLE_FORMATS:  # a table kept in 16 bits per value: the *_half entry points
             _require(lv.is_cuda, "lattice_values should be in GPU memory. Please call .cuda() on the tensor")
             _require(lv.dim() == 3, f"lattice_values should have 3 dimensions, however it has sizes {tuple(lv.shape)}")
         else:
@@ -321,11 +325,15 @@ class EncodingWrapper:
         n = pos.shape[0]
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
         out = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
-        entry = lib().penc_forward_half if lv.dtype == torch.float16 else lib().penc_forward
         with torch.cuda.device(pos.device):
-            _check(entry(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
-                         _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(out),
-                         int(fp.m_concat_points), fp.m_points_scaling, _stream()), "forward")
+            if lv.dtype in TABLE_FORMATS:
+                _check(lib().penc_forward_half(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                                               TABLE_FORMATS[lv.dtype], _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
+                                               _ptr(out), int(fp.m_concat_points), fp.m_points_scaling, _stream()), "forward")
+            else:
+                _check(lib().penc_forward(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                                          _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(out),
+                                          int(fp.m_concat_points), fp.m_points_scaling, _stream()), "forward")
         return out
 
     def backward(self, inp, grad_sliced_values_monolithic):
@@ -341,7 +349,7 @@ class EncodingWrapper:
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
         grad = grad_sliced_values_monolithic
         self._check_grad(grad, levels, extra, n, allow_rows=True)
-        half = lv.dtype == torch.float16  # the gradient w.r.t. the table is fp32 either way
+        half = lv.dtype in TABLE_FORMATS  # the gradient w.r.t. the table is fp32 either way
         lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device) if inp.m_require_lattice_values_grad else None
         pos_grad = torch.empty_like(pos) if inp.m_require_positions_grad else None
         if lv_grad is None and pos_grad is None:
@@ -351,8 +359,9 @@ class EncodingWrapper:
                 copy_bytes = 4 * self.nr_feat * levels * n + 512 if pos_grad is not None else 0
                 ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, lv_grad is not None, pos_grad is not None,
                                        fixed_bytes=copy_bytes, required_bytes=copy_bytes, nr_feat=self.nr_feat)
+                table = (_ptr(lv), TABLE_FORMATS[lv.dtype]) if half else (_ptr(lv),)
                 _check((lib().penc_backward_half if half else lib().penc_backward_rowmajor)(
-                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), *table, _ptr(fp.m_scale_factor), _ptr(shift),
                     _ptr(win), _ptr(grad), grad.stride(2), _ptr(lv_grad), _ptr(pos_grad), _ptr(ws),
                     0 if ws is None else ws.numel(), _stream()), "backward")
                 return lv_grad, pos_grad
@@ -360,7 +369,8 @@ class EncodingWrapper:
                                    nr_feat=self.nr_feat)
             if half:
                 _check(lib().penc_backward_half(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
-                                                _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(grad), 0, _ptr(lv_grad),
+                                                TABLE_FORMATS[lv.dtype], _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win),
+                                                _ptr(grad), 0, _ptr(lv_grad),
                                                 _ptr(pos_grad), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
                        "backward")
                 return lv_grad, pos_grad
@@ -386,9 +396,10 @@ class EncodingWrapper:
         ggs = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
         with torch.cuda.device(pos.device):
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, nr_feat=self.nr_feat)
-            if lv.dtype == torch.float16:
+            if lv.dtype in TABLE_FORMATS:
                 _check(lib().penc_double_backward_from_positions_half(
-                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), TABLE_FORMATS[lv.dtype],
+                    _ptr(fp.m_scale_factor), _ptr(shift),
                     _ptr(win), _ptr(dpos), _ptr(grad), 0 if grad.is_contiguous() else grad.stride(2), _ptr(lv_grad), _ptr(ggs),
                     int(fp.m_concat_points), _ptr(ws), 0 if ws is None else ws.numel(), _stream()),
                     "double_backward_from_positions")

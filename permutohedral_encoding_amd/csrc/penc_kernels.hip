@@ -45,8 +45,11 @@ __device__ __forceinline__ fvec<D> load_point(const float* __restrict__ position
 
 // The D+1 table entries of a simplex (F features each: one load of F elements per vertex, two of 16
 // bytes for eight floats), fetched back to back so that all loads are in flight together.
-// f[k][r] is feature k of vertex r.  T is the table's element type: float, or __half for a table
-// kept in half precision (the values are widened exactly; all arithmetic stays fp32).
+// f[k][r] is feature k of vertex r.  T is the table's element type: float, or __half / bfloat16_bits
+// for a table kept in 16 bits (the values are widened exactly; all arithmetic stays fp32).
+struct bfloat16_bits {
+    uint16_t bits;  // the upper half of the fp32 with the same value
+};
 template <int D, int F>
 struct Vertices {
     fvec<D + 1> f[F];
@@ -67,9 +70,14 @@ __device__ __forceinline__ Vertices<D, F> load_vertices(const T* __restrict__ le
             __builtin_memcpy(words, &raw, sizeof(raw));
             static_for<F / 2>(PENC_BODY(q) {
                 PENC_INDEX(q);
-                const float2 x = __half22float2(__builtin_bit_cast(__half2, words[q]));
-                v.f[2 * q + 0][r] = x.x;
-                v.f[2 * q + 1][r] = x.y;
+                if constexpr (std::is_same<T, bfloat16_bits>::value) {
+                    v.f[2 * q + 0][r] = __builtin_bit_cast(float, words[q] << 16);
+                    v.f[2 * q + 1][r] = __builtin_bit_cast(float, words[q] & 0xFFFF0000u);
+                } else {
+                    const float2 x = __half22float2(__builtin_bit_cast(__half2, words[q]));
+                    v.f[2 * q + 0][r] = x.x;
+                    v.f[2 * q + 1][r] = x.y;
+                }
             });
         } else if constexpr (F == 2) {
             const float2 x = *reinterpret_cast<const float2*>(level_table + 2 * slot);
@@ -541,14 +549,15 @@ inline int check_geometry(int pos_dim, int nr_feat, int64_t n, int levels, int c
 }
 
 inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
-// The table as the gathering kernels see it: fp32, or half precision (the *_half entry points).
+// The table as the gathering kernels see it: fp32 (format 0), or 16 bits per value (the *_half entry
+// points: PENC_TABLE_FP16 or PENC_TABLE_BF16).
 struct TableRef {
     const void* values;
-    bool half;
+    int format;
 };
 // a slot is gathered with one load (two of 16 bytes for eight floats): 4 to 16 bytes
 inline bool table_aligned(const TableRef& t, int nr_feat) {
-    const unsigned slot_bytes = static_cast<unsigned>(nr_feat) * (t.half ? 2u : 4u);
+    const unsigned slot_bytes = static_cast<unsigned>(nr_feat) * (t.format != 0 ? 2u : 4u);
     return (reinterpret_cast<uintptr_t>(t.values) & ((slot_bytes < 16u ? slot_bytes : 16u) - 1u)) == 0;
 }
 
@@ -686,9 +695,12 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
         PENC_DISPATCH_D(D_, __VA_ARGS__)                                \
     }
 
-// The same with the table's element type (float or __half) as TT.
-#define PENC_DISPATCH_DFT(D_, F_, HALF_, ...)                           \
-    if (HALF_) {                                                        \
+// The same with the table's element type (float, __half or bfloat16_bits) as TT.
+#define PENC_DISPATCH_DFT(D_, F_, FORMAT_, ...)                         \
+    if ((FORMAT_) == PENC_TABLE_BF16) {                                 \
+        using TT = bfloat16_bits;                                       \
+        PENC_DISPATCH_DF(D_, F_, __VA_ARGS__)                           \
+    } else if ((FORMAT_) == PENC_TABLE_FP16) {                          \
         using TT = __half;                                              \
         PENC_DISPATCH_DF(D_, F_, __VA_ARGS__)                           \
     } else {                                                            \
@@ -808,7 +820,7 @@ static int positions_backward(int pos_dim, int nr_feat, int64_t nr_positions, in
         groups = want_groups;
         partial = reinterpret_cast<float*>(ws);
     }
-    PENC_DISPATCH_DFT(pos_dim, nr_feat, table.half,
+    PENC_DISPATCH_DFT(pos_dim, nr_feat, table.format,
                       hipLaunchKernelGGL((backward_pos_kernel<DD, FF, TT>), dim3(tiles(nr_positions), groups), dim3(kBlock), 0,
                                          st, n, nr_levels, per_group, cap, mask, positions,
                                          static_cast<const TT*>(table.values), scale_factor, random_shift, anneal_window,
@@ -867,7 +879,7 @@ static int forward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_l
     if (!table_aligned(table, nr_feat)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid(tiles(nr_positions), nr_levels + extra);
-    PENC_DISPATCH_DFT(pos_dim, nr_feat, table.half,
+    PENC_DISPATCH_DFT(pos_dim, nr_feat, table.format,
                       hipLaunchKernelGGL((forward_kernel<DD, FF, TT>), grid, dim3(kBlock), 0, st,
                                          static_cast<int>(nr_positions), nr_levels, static_cast<uint32_t>(capacity),
                                          mask_of(capacity), positions, static_cast<const TT*>(table.values), scale_factor,
@@ -887,6 +899,7 @@ const char* penc_status_string(int status) {
         case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to one slot (at most 16 bytes), lattice_values_grad and gradient rows to 8 bytes";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
         case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major copy of the upstream gradient (penc_backward_rowmajor_workspace_bytes)";
+        case PENC_ERR_UNSUPPORTED_TABLE_FORMAT: return "table_format must be PENC_TABLE_FP16 or PENC_TABLE_BF16";
         case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
         default: return "unknown status";
     }
@@ -938,15 +951,16 @@ int penc_forward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, 
                  const float* positions, const float* lattice_values, const float* scale_factor,
                  const float* random_shift, const float* anneal_window, float* sliced_values,
                  int concat_points, float points_scaling, void* stream) {
-    return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+    return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                         scale_factor, random_shift, anneal_window, sliced_values, concat_points, points_scaling, stream);
 }
 
 int penc_forward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                      const float* positions, const void* lattice_values_half, const float* scale_factor,
-                      const float* random_shift, const float* anneal_window, float* sliced_values,
-                      int concat_points, float points_scaling, void* stream) {
-    return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values_half, true},
+                      const float* positions, const void* lattice_values_half, int table_format,
+                      const float* scale_factor, const float* random_shift, const float* anneal_window,
+                      float* sliced_values, int concat_points, float points_scaling, void* stream) {
+    if (table_format != PENC_TABLE_FP16 && table_format != PENC_TABLE_BF16) return PENC_ERR_UNSUPPORTED_TABLE_FORMAT;
+    return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values_half, table_format},
                         scale_factor, random_shift, anneal_window, sliced_values, concat_points, points_scaling, stream);
 }
 
@@ -955,7 +969,7 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
                   const float* random_shift, const float* anneal_window,
                   const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
                   void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                          scale_factor, random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad,
                          workspace, workspace_bytes, stream);
 }
@@ -975,7 +989,7 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
         return PENC_ERR_SCRATCH_TOO_SMALL;
     void* ws = static_scratch_of_current_device();
     if (ws == nullptr) return PENC_ERR_LAUNCH;
-    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                          scale_factor, random_shift, anneal_window, grad_sliced_values, lattice_values_grad, positions_grad, ws,
                          PENC_STATIC_SCRATCH_BYTES, stream);
 }
@@ -1048,17 +1062,18 @@ int penc_backward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int n
                            const float* random_shift, const float* anneal_window, const float* grad_rows,
                            int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
                            void* workspace, size_t workspace_bytes, void* stream) {
-    return backward_rowmajor_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+    return backward_rowmajor_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                                   scale_factor, random_shift, anneal_window, grad_rows, grad_row_stride, lattice_values_grad,
                                   positions_grad, workspace, workspace_bytes, stream);
 }
 
 int penc_backward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                       const float* positions, const void* lattice_values_half, const float* scale_factor,
-                       const float* random_shift, const float* anneal_window, const float* grad,
-                       int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
+                       const float* positions, const void* lattice_values_half, int table_format,
+                       const float* scale_factor, const float* random_shift, const float* anneal_window,
+                       const float* grad, int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
                        void* workspace, size_t workspace_bytes, void* stream) {
-    const TableRef table{lattice_values_half, true};
+    if (table_format != PENC_TABLE_FP16 && table_format != PENC_TABLE_BF16) return PENC_ERR_UNSUPPORTED_TABLE_FORMAT;
+    const TableRef table{lattice_values_half, table_format};
     if (grad_row_stride != 0)
         return backward_rowmajor_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor,
                                       random_shift, anneal_window, grad, grad_row_stride, lattice_values_grad, positions_grad,
@@ -1093,7 +1108,7 @@ static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, 
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (grad_grad_sliced_values) {
         const dim3 grid(tiles(nr_positions), nr_levels + extra);
-        PENC_DISPATCH_DFT(pos_dim, nr_feat, table.half,
+        PENC_DISPATCH_DFT(pos_dim, nr_feat, table.format,
                           hipLaunchKernelGGL((grad_grad_kernel<DD, FF, TT>), grid, dim3(kBlock), 0, st,
                                              static_cast<int>(nr_positions), nr_levels, static_cast<uint32_t>(capacity),
                                              mask_of(capacity), positions, static_cast<const TT*>(table.values), scale_factor,
@@ -1114,7 +1129,7 @@ int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_pos
                                         const float* grad_sliced_values, float* lattice_values_grad,
                                         float* grad_grad_sliced_values, int concat_points, void* workspace,
                                         size_t workspace_bytes, void* stream) {
-    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                                 scale_factor, random_shift, anneal_window, double_positions_grad, grad_sliced_values, 0,
                                 lattice_values_grad, grad_grad_sliced_values, concat_points, workspace, workspace_bytes,
                                 stream);
@@ -1130,23 +1145,24 @@ int penc_double_backward_from_positions_rowmajor(int pos_dim, int nr_feat, int64
                                                  void* stream) {
     if (nr_levels > 0 && nr_positions > 0)
         if (int rc = check_rows(grad_rows, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
-    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, false},
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                                 scale_factor, random_shift, anneal_window, double_positions_grad, grad_rows,
                                 grad_row_stride, lattice_values_grad, grad_grad_sliced_values, concat_points, workspace,
                                 workspace_bytes, stream);
 }
 
 int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
-                                             const float* positions, const void* lattice_values_half,
+                                             const float* positions, const void* lattice_values_half, int table_format,
                                              const float* scale_factor, const float* random_shift,
                                              const float* anneal_window, const float* double_positions_grad,
                                              const float* grad, int64_t grad_row_stride, float* lattice_values_grad,
                                              float* grad_grad_sliced_values, int concat_points, void* workspace,
                                              size_t workspace_bytes, void* stream) {
+    if (table_format != PENC_TABLE_FP16 && table_format != PENC_TABLE_BF16) return PENC_ERR_UNSUPPORTED_TABLE_FORMAT;
     if (grad_row_stride != 0 && nr_levels > 0 && nr_positions > 0)
         if (int rc = check_rows(grad, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
     return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions,
-                                TableRef{lattice_values_half, true}, scale_factor, random_shift, anneal_window,
+                                TableRef{lattice_values_half, table_format}, scale_factor, random_shift, anneal_window,
                                 double_positions_grad, grad, grad_row_stride, lattice_values_grad, grad_grad_sliced_values,
                                 concat_points, workspace, workspace_bytes, stream);
 }

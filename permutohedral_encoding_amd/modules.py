@@ -15,17 +15,26 @@ class PermutoEncoding(torch.nn.Module):
     Same constructor, parameters (``lattice_values`` (L, C, F), ``random_shift_per_level`` (L, D)) and
     forward as the reference module (modules.py:10-103).  Two additions: ``device`` defaults to the
     current GPU (a CPU device is accepted for construction only: the forward has no CPU path), and
-    ``lattice_half_precision=True`` makes the kernels gather from a half-precision copy of
-    ``lattice_values`` (the switch the reference carries disabled, EncodingGPU.cuh:12).  The
-    parameter itself and every gradient stay fp32; the copy is refreshed whenever the parameter has
-    been modified in place (optimizer steps), so it pays for large tables and for inference.
+    ``lattice_half_precision`` (``True`` or ``torch.float16``, or ``torch.bfloat16``) makes the
+    kernels gather from a 16-bit copy of ``lattice_values`` (the switch the reference carries
+    disabled, EncodingGPU.cuh:12).  The parameter itself and every gradient stay fp32; the copy is
+    refreshed whenever the parameter has been modified in place (optimizer steps), so it pays for
+    large tables and for inference.  float16 resolves the reference's initial values (about 1e-5)
+    only to 6e-8; bfloat16 keeps three significant digits at any magnitude.
     """
 
     def __init__(self, pos_dim, capacity, nr_levels, nr_feat_per_level, scale_per_level,
                  appply_random_shift_per_level=True, concat_points=False, concat_points_scaling=1.0, device=None,
                  lattice_half_precision=False):
         super().__init__()
-        self.lattice_half_precision = bool(lattice_half_precision)
+        if lattice_half_precision in (None, False):
+            self.lattice_half_precision = None
+        elif lattice_half_precision is True or lattice_half_precision == torch.float16:
+            self.lattice_half_precision = torch.float16
+        elif lattice_half_precision == torch.bfloat16:
+            self.lattice_half_precision = torch.bfloat16
+        else:
+            raise ValueError("lattice_half_precision must be False, True, torch.float16 or torch.bfloat16")
         self.pos_dim = pos_dim
         self.capacity = capacity
         self.nr_levels = nr_levels
@@ -64,7 +73,7 @@ class PermutoEncoding(torch.nn.Module):
                                                    self.scale_per_level, self.random_shift_per_level,
                                                    self.concat_points, self.concat_points_scaling)
         lattice = _native.EncodingWrapper.create(self.pos_dim, self.nr_feat_per_level, fixed_params)
-        lattice.half_table = getattr(self, "lattice_half_precision", False)
+        lattice.half_table = getattr(self, "lattice_half_precision", None)
         return fixed_params, lattice
 
     def __getstate__(self):

@@ -366,20 +366,22 @@ def test_module_with_more_features_per_level(feat):
     assert np.all(err <= 1e-4 * r["abs64"] + 1e-30)
 
 
-def test_module_gathers_from_a_half_precision_copy():
-    """PermutoEncoding(..., lattice_half_precision=True): the kernels gather from a float16 copy of the
-    fp32 parameter; the output is that of the rounded table, gradients reach the fp32 parameter in fp32
-    (first and second order), and the copy follows in-place updates of the parameter."""
+@pytest.mark.parametrize("switch,dtype", [(True, torch.float16), (torch.float16, torch.float16), (torch.bfloat16, torch.bfloat16)])
+def test_module_gathers_from_a_half_precision_copy(switch, dtype):
+    """PermutoEncoding(..., lattice_half_precision=True or a 16-bit dtype): the kernels gather from a 16-bit
+    copy of the fp32 parameter; the output is that of the rounded table, gradients reach the fp32 parameter
+    in fp32 (first and second order), and the copy follows in-place updates of the parameter."""
     import permutohedral_encoding_amd as pe
     torch.manual_seed(3)
     levels, n = 5, 2000
-    m = pe.PermutoEncoding(3, 1 << 12, levels, 2, np.geomspace(1.0, 1e-2, levels), lattice_half_precision=True)
+    m = pe.PermutoEncoding(3, 1 << 12, levels, 2, np.geomspace(1.0, 1e-2, levels), lattice_half_precision=switch)
+    narrow = lambda a: torch.from_numpy(a).to(dtype).to(torch.float32).numpy()
     with torch.no_grad():
         m.lattice_values.uniform_(-1, 1)
     pos = torch.rand(n, 3, device="cuda", requires_grad=True)
     out = m(pos)
     p, t, sf, sh = oracle_args(m, pos)
-    rounded = t.astype(np.float16).astype(np.float32)
+    rounded = narrow(t)
     assert not np.array_equal(rounded, t)
     w = np.ones(levels, np.float32)
     want = orc.forward(p, rounded, sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
@@ -398,12 +400,12 @@ def test_module_gathers_from_a_half_precision_copy():
     with torch.no_grad():
         m.lattice_values.mul_(0.5)
     out2 = m(pos.detach())
-    want2 = orc.forward(p, (0.5 * t).astype(np.float16).astype(np.float32), sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
+    want2 = orc.forward(p, narrow(0.5 * t), sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
     assert np.array_equal(out2.detach().cpu().numpy(), want2)
     # pickling keeps the switch
     import pickle
     m2 = pickle.loads(pickle.dumps(m))
-    assert m2.lattice_half_precision and torch.equal(m2(pos.detach()), out2)
+    assert m2.lattice_half_precision == dtype and torch.equal(m2(pos.detach()), out2)
 
 
 @pytest.mark.parametrize("n", [4096, 4099, 3])

@@ -234,10 +234,11 @@ def test_more_features_at_benchmark_size_with_rows_and_concat_points(feat, n):
 
 # ----------------------------------------------------------------------------- table in half precision
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("feat", [2, 4, 8])
 @pytest.mark.parametrize("d", [2, 3, 4, 8])
-def test_half_precision_table_equals_the_widened_table(d, feat):
-    """A float16 table through the *_half entry points: the kernels widen on load and compute in fp32, so
+def test_half_precision_table_equals_the_widened_table(d, feat, dtype):
+    """A float16 or bfloat16 table through the *_half entry points: the kernels widen on load and compute in fp32, so
     every result is that of the fp32 path on the widened table: forward and grad-of-grad bit-equal to the
     oracle run on it, position gradient within its bound, table gradients (which never read the table)
     fp32 as before.  Level-major and row-major upstream gradients."""
@@ -245,12 +246,12 @@ def test_half_precision_table_equals_the_widened_table(d, feat):
     cap = (1 << 12) if d != 3 else 5001  # odd capacity: slots of 2F bytes at odd offsets
     n, levels = 5000, 4
     p = random_problem(d, n, levels, cap, seed=130 + d + feat, sigma_range=(1.0, 1e-3), nr_feat=feat)
-    half = p["table"].astype(np.float16)
-    p["table"] = half.astype(np.float32)
+    half = torch.from_numpy(p["table"]).to(dtype)  # rounded by torch: the conversion a caller would use
+    p["table"] = half.to(torch.float32).numpy()
     sf = orc.scale_factors(d, p["sigmas"])
     enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
     inp = gpu_input(p)
-    inp.m_lattice_values = to_gpu(half)
+    inp.m_lattice_values = half.cuda()
     out = enc.forward(inp).cpu().numpy()
     assert np.array_equal(out, orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"]))
     rows = to_gpu(np.ascontiguousarray(p["grad"].transpose(2, 0, 1).reshape(n, levels * feat)))

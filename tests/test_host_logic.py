@@ -70,12 +70,16 @@ def test_argument_validation_without_a_gpu():
     assert lib.penc_double_backward_from_positions(3, 2, 10, 2, 16, p, p, p, p, p, p, p, z, z, 0, None, 0, None) == 1
     assert lib.penc_simplex_debug(3, 0, 2, 16, p, p, p, 0, z, z, z, z, None) == 2
     # a table in half precision: slots of 2F bytes (4 for two features, 16 for eight)
-    assert lib.penc_forward_half(3, 2, 10, 2, 16, p, p + 2, p, p, p, p, 0, 1.0, None) == 5
-    assert lib.penc_forward_half(3, 8, 10, 2, 16, p, p + 8, p, p, p, p, 0, 1.0, None) == 5
-    assert lib.penc_forward_half(3, 2, 10, 2, 16, p, z, p, p, p, p, 0, 1.0, None) == 1
-    assert lib.penc_backward_half(3, 2, 10, 2, 16, p, z, p, p, p, p, 0, z, p, None, 0, None) == 1  # position gradient needs the table
-    assert lib.penc_backward_half(3, 2, 10, 2, 16, p, p, p, p, p, p, 3, p, z, None, 0, None) == 2  # odd row stride
-    assert lib.penc_double_backward_from_positions_half(3, 2, 10, 2, 16, p, p, p, p, p, p, p, 0, z, z, 0, None, 0, None) == 1
+    assert lib.penc_forward_half(3, 2, 10, 2, 16, p, p + 2, 1, p, p, p, p, 0, 1.0, None) == 5
+    assert lib.penc_forward_half(3, 8, 10, 2, 16, p, p + 8, 2, p, p, p, p, 0, 1.0, None) == 5
+    assert lib.penc_forward_half(3, 2, 10, 2, 16, p, z, 1, p, p, p, p, 0, 1.0, None) == 1
+    assert lib.penc_forward_half(3, 2, 10, 2, 16, p, p, 0, p, p, p, p, 0, 1.0, None) == 9  # neither binary16 nor bfloat16
+    assert lib.penc_forward_half(3, 2, 10, 2, 16, p, p, 3, p, p, p, p, 0, 1.0, None) == 9
+    assert lib.penc_backward_half(3, 2, 10, 2, 16, p, z, 1, p, p, p, p, 0, z, p, None, 0, None) == 1  # position gradient needs the table
+    assert lib.penc_backward_half(3, 2, 10, 2, 16, p, p, 2, p, p, p, p, 3, p, z, None, 0, None) == 2  # odd row stride
+    assert lib.penc_backward_half(3, 2, 10, 2, 16, p, p, 7, p, p, p, p, 0, p, z, None, 0, None) == 9
+    assert lib.penc_double_backward_from_positions_half(3, 2, 10, 2, 16, p, p, 1, p, p, p, p, p, 0, z, z, 0, None, 0, None) == 1
+    assert lib.penc_double_backward_from_positions_half(3, 2, 10, 2, 16, p, p, 0, p, p, p, p, p, 0, p, p, 0, None, 0, None) == 9
     # the optimizer step
     assert lib.penc_adamw_step(z, p, p, p, 16, 1e-3, 0.9, 0.99, 1e-8, 0.0, 1, 0, None) == 1
     assert lib.penc_adamw_step(p, p, p, p, 0, 1e-3, 0.9, 0.99, 1e-8, 0.0, 1, 0, None) == 2
