@@ -565,10 +565,9 @@ __device__ __forceinline__ void column_tile(State& c, const GradSlice& level_gra
     });
 }
 
-// Sums every column in use and sends the sums on to stage 2 (or 3).  By all threads, between barriers.
+// Sums every column in use and adds the sums to the gradient (stage 3).  By all threads, between barriers.
 template <typename State>
-__device__ __forceinline__ void column_flush(State& c, const GradSlice& level_grad, const BinTarget& bins,
-                                             uint32_t group, uint32_t id_bits) {
+__device__ __forceinline__ void column_flush(State& c, const GradSlice& level_grad, uint32_t id_bits) {
     const uint32_t cell_bits = kCacheLinesLog2 - id_bits, cells = 1u << cell_bits;
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     for (uint32_t id = wave; id < (1u << id_bits); id += kScatterBlock / 64) {
@@ -582,13 +581,11 @@ __device__ __forceinline__ void column_flush(State& c, const GradSlice& level_gr
             s1 += __shfl_xor(s1, step);
         }
         if (lane == 0) {
-            const float v0 = static_cast<float>(s0), v1 = static_cast<float>(s1);
-            const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
-            if (!binned) {
-                float* g = level_grad.at(static_cast<uint32_t>(owner));
-                global_add(g, v0);
-                global_add(g + 1, v1);
-            }
+            // straight into the gradient: a level in column mode leaves a few dozen sums per workgroup, and
+            // as records they would only make every bin's reducer workgroup run for a handful of them
+            float* g = level_grad.at(static_cast<uint32_t>(owner));
+            global_add(g, static_cast<float>(s0));
+            global_add(g + 1, static_cast<float>(s1));
         }
     }
 }
@@ -740,7 +737,7 @@ __device__ __forceinline__ void scatter_end(State& c, const GradSlice& level_gra
                                             uint32_t group, int mode, uint32_t id_bits) {
     __syncthreads();
     if (mode == kModeCache) cache_flush(c, level_grad, bins, group);
-    if (mode == kModeColumns) column_flush(c, level_grad, bins, group, id_bits);
+    if (mode == kModeColumns) column_flush(c, level_grad, id_bits);
     if (bins.records == nullptr) return;
     __syncthreads();
     for (uint32_t b = threadIdx.x; b < bins.n_bins; b += kScatterBlock) {
@@ -774,11 +771,6 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     const uint32_t level = pair_level / feat_pairs, pair = pair_level % feat_pairs;
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
-    for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
-        acc0[s] = 0.0;
-        acc1[s] = 0.0;
-    }
-    __syncthreads();
     constexpr uint32_t kWaves = kReduceBlock / 64;
     constexpr uint32_t kUnroll = 4;
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -787,6 +779,16 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     const uint32_t group_end = group_begin + per_split < bins.n_groups ? group_begin + per_split : bins.n_groups;
     const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
     const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
+    // A bin nothing was appended to (the levels whose scattering workgroups summed in columns, a slot
+    // range no point touches) ends here: the look at the counts overlaps the clearing of the sums,
+    // and the barrier that follows the clearing carries the vote.
+    bool any = false;
+    for (uint32_t g = group_begin + threadIdx.x; g < group_end; g += kReduceBlock) any = any || counts[g] != 0u;
+    for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
+        acc0[s] = 0.0;
+        acc1[s] = 0.0;
+    }
+    if (!__syncthreads_or(any)) return;
     // segments g = group_begin + wave, + kWaves, ...; their record counts are fetched 64 at a time
     // (one per lane) so that no segment has to wait for its own count.  The records are walked in
     // chunks of kUnroll wave-widths, and the next chunk's loads are issued before the current
