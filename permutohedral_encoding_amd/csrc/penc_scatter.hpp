@@ -984,19 +984,40 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs};
     const uint32_t slot0 = bin << kBinSlotsLog2;
     const bool alone = gridDim.z == 1;
+    if (alone) {
+        // all of a thread's read-modify-writes at once: the loads are issued together, not one per trip
+        constexpr int kMine = kBinSlots / kReduceBlock;
+        float2 sum[kMine], g[kMine];
+        bool touched[kMine];
+#pragma unroll
+        for (int k = 0; k < kMine; ++k) {
+            const uint32_t s = static_cast<uint32_t>(k) * kReduceBlock + threadIdx.x;
+            const double v0 = acc0[s], v1 = acc1[s];
+            sum[k] = make_float2(static_cast<float>(v0), static_cast<float>(v1));
+            touched[k] = (v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity;
+        }
+#pragma unroll
+        for (int k = 0; k < kMine; ++k) {
+            const uint32_t s = static_cast<uint32_t>(k) * kReduceBlock + threadIdx.x;
+            if (touched[k]) g[k] = *reinterpret_cast<const float2*>(level_grad.at(slot0 + s));
+        }
+#pragma unroll
+        for (int k = 0; k < kMine; ++k) {
+            const uint32_t s = static_cast<uint32_t>(k) * kReduceBlock + threadIdx.x;
+            if (touched[k]) {
+                g[k].x += sum[k].x;
+                g[k].y += sum[k].y;
+                *reinterpret_cast<float2*>(level_grad.at(slot0 + s)) = g[k];
+            }
+        }
+        return;
+    }
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
         const double v0 = acc0[s], v1 = acc1[s];
         if ((v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity) {
             float2* cell = reinterpret_cast<float2*>(level_grad.at(slot0 + s));
-            if (alone) {
-                float2 g = *cell;
-                g.x += static_cast<float>(v0);
-                g.y += static_cast<float>(v1);
-                *cell = g;
-            } else {
-                global_add(&cell->x, static_cast<float>(v0));
-                global_add(&cell->y, static_cast<float>(v1));
-            }
+            global_add(&cell->x, static_cast<float>(v0));
+            global_add(&cell->y, static_cast<float>(v1));
         }
     }
 }
