@@ -726,6 +726,19 @@ def test_table_gradients_on_mixed_point_distributions(seed):
     _table_gradients_match(p, d, cap, f"seed {seed}: D={d} cap={cap} n={n} clusters={n_clusters}")
 
 
+def test_segments_overflow_with_more_bins_than_lanes():
+    """The same deception on a 2^20-slot table (128 slot ranges: the tile is sorted with one counter and
+    one thread per bin): the first 512 points of every group are spread out, all the others sit in one
+    simplex, so thousands of records head for a few segments sized for a few hundred."""
+    d, n, levels, cap = 3, 6 * 8192 + 777, 5, 1 << 20
+    rng = np.random.default_rng(123)
+    p = random_problem(d, n, levels, cap, seed=124, sigma_range=(1.0, 1e-3))
+    clustered = (np.arange(n) % 4096) >= 512
+    cluster = (0.61 + 1e-7 * rng.standard_normal((n, d))).astype(np.float32)
+    p["pos"] = np.where(clustered[:, None], cluster, p["pos"]).astype(np.float32)
+    _table_gradients_match(p, d, cap, "segments overflow, 128 bins")
+
+
 def test_records_crowd_one_bin():
     """Points chosen so that, at the finest level, at least three of their four vertices fall into the
     first of four slot ranges: the tile's records are all distinct (the workgroup streams them sorted
