@@ -75,8 +75,9 @@ int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* s
  * is too large for binning (above 2^22 slots).  `nr_levels` counts pairs of features: pass
  * nr_levels * nr_feat / 2.  Per level the workspace holds, for each of the ceil(capacity / 8192)
  * slot ranges and each group of 4096 or 8192 points, a 4-byte count and room for the group's
- * expected share of the (pos_dim + 1) 12-byte records per point plus three standard deviations:
- * about 13.5 * (pos_dim + 1) bytes per point and level (1.4 GiB for 2^20 points, 24 levels, pos_dim 3).
+ * expected share of the (pos_dim + 1) records per point plus three standard deviations; a record is
+ * 10 bytes for pos_dim <= 5 and capacities up to 2^19 and 12 bytes otherwise: about 11.5 or
+ * 13.5 * (pos_dim + 1) bytes per point and level (1.2 GiB for 2^20 points, 24 levels, pos_dim 3).
  * Any smaller workspace works too: the levels are then binned in several passes, and with none the
  * gradient is accumulated with direct atomics.  No counterpart in the reference (its scatter is one
  * atomicAdd per value, EncodingGPU.cuh:409-410). */

@@ -603,17 +603,25 @@ inline int table_backward_tiles(int64_t n, int levels) {
                                                                                                             : kScatterTiles;
 }
 
-// Records one scattering workgroup may leave in one bin: its share of the group's
+// Split records (10 bytes in two arrays) where a tile's records leave in long runs (the
+// workgroup-wide sort), whole ones (12 bytes) elsewhere (see BinRecord).
+inline size_t record_bytes(int pos_dim, uint32_t n_bins) {
+    return pos_dim <= kWorkgroupSortMaxDim && n_bins <= static_cast<uint32_t>(kStageBins) ? kSplitRecordBytes : sizeof(BinRecord);
+}
+
+// Records one scattering workgroup may leave in one bin: its share of the
 // group's contributions (D+1 per point) plus the flushed cache lines, with three standard deviations
 // of a uniform hash on top.  A segment that still overflows spills to direct atomics.
 inline uint32_t wanted_segment_capacity(int pos_dim, uint32_t n_bins, int tiles_per_group) {
     const double mean = (static_cast<double>(tiles_per_group) * kScatterBlock * (pos_dim + 1) + kCacheLines) / n_bins;
-    return static_cast<uint32_t>(mean + 3.0 * __builtin_sqrt(mean) + 8.0);
+    const uint32_t cap = static_cast<uint32_t>(mean + 3.0 * __builtin_sqrt(mean) + 8.0);
+    // split records: a multiple of four per segment keeps every segment's values 16-byte aligned
+    return record_bytes(pos_dim, n_bins) == kSplitRecordBytes ? (cap + 3u) & ~3u : cap;
 }
 
-inline size_t bin_bytes_per_level(uint32_t n_bins, uint32_t n_groups, uint32_t segment_capacity) {
+inline size_t bin_bytes_per_level(int pos_dim, uint32_t n_bins, uint32_t n_groups, uint32_t segment_capacity) {
     const size_t segments = static_cast<size_t>(n_bins) * n_groups;
-    return segments * (sizeof(uint32_t) + static_cast<size_t>(segment_capacity) * sizeof(BinRecord));
+    return segments * (sizeof(uint32_t) + static_cast<size_t>(segment_capacity) * record_bytes(pos_dim, n_bins));
 }
 
 inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int tiles_per_group, void* workspace,
@@ -630,25 +638,30 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int t
     if (bytes < lost + 4096) return p;
     bytes -= lost + 256;
     const size_t segments = static_cast<size_t>(n_bins) * n_groups;
+    const bool split = record_bytes(pos_dim, n_bins) == kSplitRecordBytes;
     uint32_t cap = wanted_segment_capacity(pos_dim, n_bins, tiles_per_group);
-    if (bytes < bin_bytes_per_level(n_bins, n_groups, cap)) {  // not even one level at the wanted size: shrink the segments
-        if (bytes < segments * (sizeof(uint32_t) + 16 * sizeof(BinRecord))) return p;
-        cap = static_cast<uint32_t>((bytes / segments - sizeof(uint32_t)) / sizeof(BinRecord));
+    if (bytes < bin_bytes_per_level(pos_dim, n_bins, n_groups, cap)) {  // not even one level at the wanted size: shrink the segments
+        if (bytes < segments * (sizeof(uint32_t) + 16 * record_bytes(pos_dim, n_bins))) return p;
+        cap = static_cast<uint32_t>((bytes / segments - sizeof(uint32_t)) / record_bytes(pos_dim, n_bins));
+        if (split) cap &= ~3u;
     }
     // the scattering kernel addresses a level's records with 32-bit byte offsets
-    constexpr uint64_t kMaxRecordsPerLevel = 0xFFFFFFFFull / sizeof(BinRecord);
-    if (segments * cap > kMaxRecordsPerLevel) {
-        cap = static_cast<uint32_t>(kMaxRecordsPerLevel / segments);
+    const uint64_t max_records_per_level = 0xFFFFFFFFull / (split ? sizeof(RecordValues) : sizeof(BinRecord));
+    if (segments * cap > max_records_per_level) {
+        cap = static_cast<uint32_t>(max_records_per_level / segments);
+        if (split) cap &= ~3u;
         if (cap < 16) return p;
     }
-    const size_t fit = bytes / bin_bytes_per_level(n_bins, n_groups, cap);
+    const size_t fit = bytes / bin_bytes_per_level(pos_dim, n_bins, n_groups, cap);
     p.levels_per_pass = static_cast<int>(fit < static_cast<size_t>(levels) ? fit : static_cast<size_t>(levels));
     p.target.n_bins = n_bins;
     p.target.n_groups = n_groups;
     p.target.segment_capacity = cap;
     p.target.counts = reinterpret_cast<uint32_t*>(base);
     const size_t counts_bytes = (static_cast<size_t>(p.levels_per_pass) * segments * sizeof(uint32_t) + 255u) & ~size_t{255};
-    p.target.records = reinterpret_cast<BinRecord*>(base + counts_bytes);
+    const size_t records_per_pass = static_cast<size_t>(p.levels_per_pass) * segments * cap;
+    p.target.records = reinterpret_cast<void*>(base + counts_bytes);
+    p.target.slots = split ? reinterpret_cast<uint16_t*>(base + counts_bytes + records_per_pass * sizeof(RecordValues)) : nullptr;
     p.enabled = true;
     return p;
 }
@@ -665,8 +678,13 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
     unsigned splits = pairs >= kReduceWorkgroupsWanted ? 1u : (kReduceWorkgroupsWanted + pairs - 1) / pairs;
     if (splits > p.target.n_groups) splits = p.target.n_groups;
     if (splits > kMaxReduceSplits) splits = kMaxReduceSplits;
-    hipLaunchKernelGGL(bin_reduce_kernel, dim3(p.target.n_bins, n_levels_in_pass, splits), dim3(kReduceBlock), 0, st,
-                       p.target, window, static_cast<uint32_t>(capacity), feat_pairs, table_grad, first_level);
+    const dim3 grid(p.target.n_bins, n_levels_in_pass, splits);
+    if (p.target.slots != nullptr)
+        hipLaunchKernelGGL(bin_reduce_kernel<true>, grid, dim3(kReduceBlock), 0, st, p.target, window,
+                           static_cast<uint32_t>(capacity), feat_pairs, table_grad, first_level);
+    else
+        hipLaunchKernelGGL(bin_reduce_kernel<false>, grid, dim3(kReduceBlock), 0, st, p.target, window,
+                           static_cast<uint32_t>(capacity), feat_pairs, table_grad, first_level);
     return check_launch();
 }
 
@@ -919,7 +937,7 @@ size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_le
     // the larger of what the two gradient calls plan for (they may group the points differently)
     size_t per_level = 0;
     for (const int tiles : {kScatterTiles, table_backward_tiles(nr_positions, nr_levels)}) {
-        const size_t need = bin_bytes_per_level(n_bins, scatter_groups(nr_positions, tiles),
+        const size_t need = bin_bytes_per_level(pos_dim, n_bins, scatter_groups(nr_positions, tiles),
                                                 wanted_segment_capacity(pos_dim, n_bins, tiles));
         per_level = need > per_level ? need : per_level;
     }

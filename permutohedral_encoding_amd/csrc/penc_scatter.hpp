@@ -63,38 +63,40 @@ enum ScatterMode : int { kModeCache = 0, kModeStream = 1, kModeColumns = 2 };
 // vertices per thread a wave sorts by bin in one go (256 or 320 records): all D+1 of them up to D = 4
 constexpr int stage_chunk(int pos_dim) { return pos_dim + 1 <= 4 ? 4 : 5; }
 constexpr int kStageBins = 64;         // a wave counts one bin per lane: staging needs n_bins <= 64
+constexpr int kWorkgroupSortMaxDim = 5;  // up to this input dimension a streaming workgroup sorts a tile's records across all its waves
 constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
 constexpr int kMaxBins = 512;          // bins per level; capacities above kMaxBins*kBinSlots (2^22) are not binned
 constexpr int kReduceBlock = 1024;     // threads of a bin_reduce_kernel workgroup
 
+// A contribution on its way through a bin: the slot within the bin's range and the two values.
+// In memory the records of a level are either one array of these 12-byte structures, or 10 bytes in
+// two arrays indexed alike, the values (8 bytes) and the slots (2 bytes: a bin spans 2^13 slots).
+// The fine levels move nothing but records through the HBM, twice, so the split form saves a sixth
+// of their traffic (measured on a 2^18-slot table: the reducer 0.163 -> 0.150 ms, the scattering
+// kernel unchanged); it takes two stores per record, which pays only where a tile's records leave in long
+// runs, i.e. where the workgroup-wide sort of stream_tile applies (measured on a 2^22-slot table, whose runs are
+// about four records: the scattering kernel 0.313 -> 0.355 ms, the reducer 0.207 -> 0.218 ms; at
+// D = 8, whose waves sort on their own and leave runs of eight: 0.343 -> 0.356 ms, 0.137 -> 0.129 ms).
 struct BinRecord {
     uint32_t slot_in_bin;
     float a0, a1;
 };
-// A record read with the non-temporal hint: the reducer reads every record once, and a normal
-// load would make room for it in the caches by evicting records the scatter has just written and
-// that are still waiting there to be read (measured: the reducer of 2^18-slot tables 0.213 ->
-// 0.168 ms; non-temporal *stores* of the records cost the scatter more than they save here).
+static_assert(kBinSlotsLog2 <= 16, "a split record keeps its slot within the bin in 16 bits");
+typedef float RecordValues __attribute__((ext_vector_type(2)));
 typedef uint32_t RecordWords __attribute__((ext_vector_type(3), aligned(4)));
-__device__ __forceinline__ BinRecord load_record_once(const BinRecord* from) {
-    const RecordWords w = __builtin_nontemporal_load(reinterpret_cast<const RecordWords*>(from));
-    const uint32_t w0 = w.x, w1 = w.y, w2 = w.z;  // copies first: a bit cast applied directly to a vector element reads element 0
-    BinRecord rec;
-    rec.slot_in_bin = w0;
-    rec.a0 = __builtin_bit_cast(float, w1);
-    rec.a1 = __builtin_bit_cast(float, w2);
-    return rec;
-}
+constexpr size_t kSplitRecordBytes = sizeof(RecordValues) + sizeof(uint16_t);
 
 // Where the misses of the levels of one launch go.  Every scattering workgroup (a "group" of
 // points at one level) owns a private segment of `segment_capacity` records in every
 // bin, so appending needs no global atomics and no synchronisation: the cursor is an LDS counter.
-//   records [level_in_pass][bin][group][segment_capacity]
+//   records [level_in_pass][bin][group][segment_capacity]   12-byte records, or the 8-byte values of split ones
+//   slots   [level_in_pass][bin][group][segment_capacity]   the 2-byte slots of split records; nullptr otherwise
 //   counts  [level_in_pass][bin][group]            records actually written (<= segment_capacity)
 // `records` == nullptr disables binning.
 struct BinTarget {
-    BinRecord* records;
+    void* records;
+    uint16_t* slots;
     uint32_t* counts;
     uint32_t n_bins;
     uint32_t n_groups;
@@ -106,10 +108,67 @@ __device__ __forceinline__ BinTarget bins_of_level(const BinTarget& pass, uint32
     BinTarget t = pass;
     if (pass.records != nullptr) {
         const size_t segments = static_cast<size_t>(k) * pass.n_bins * pass.n_groups;
-        t.records += segments * pass.segment_capacity;
+        const size_t records = segments * pass.segment_capacity;
+        t.records = static_cast<char*>(pass.records) + records * (pass.slots != nullptr ? sizeof(RecordValues) : sizeof(BinRecord));
+        if (pass.slots != nullptr) t.slots += records;
         t.counts += segments;
     }
     return t;
+}
+
+// Writes record `i` of a level (32-bit byte offsets: the host plans for that).
+__device__ __forceinline__ void store_record(const BinTarget& bins, uint32_t i, uint32_t slot_in_bin, float a0, float a1) {
+    char* const bytes = static_cast<char*>(bins.records);
+    if (bins.slots != nullptr) {
+        RecordValues v;
+        v.x = a0;
+        v.y = a1;
+        *reinterpret_cast<RecordValues*>(bytes + i * static_cast<uint32_t>(sizeof(RecordValues))) = v;
+        *reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(bins.slots) + i * 2u) = static_cast<uint16_t>(slot_in_bin);
+    } else {
+        BinRecord rec;
+        rec.slot_in_bin = slot_in_bin;
+        rec.a0 = a0;
+        rec.a1 = a1;
+        *reinterpret_cast<BinRecord*>(bytes + i * static_cast<uint32_t>(sizeof(BinRecord))) = rec;
+    }
+}
+
+// Record `i` of a bin whose first record is `first` (of the level's arrays), with ordinary loads.
+template <bool kSplit>
+__device__ __forceinline__ BinRecord load_record(const BinTarget& bins, size_t first, uint32_t i) {
+    BinRecord rec;
+    if constexpr (kSplit) {
+        const RecordValues v = static_cast<const RecordValues*>(bins.records)[first + i];
+        rec.slot_in_bin = bins.slots[first + i];
+        rec.a0 = v.x;
+        rec.a1 = v.y;
+    } else {
+        rec = static_cast<const BinRecord*>(bins.records)[first + i];
+    }
+    return rec;
+}
+
+// The same with the non-temporal hint: the reducer reads every record once, and a normal
+// load would make room for it in the caches by evicting records the scatter has just written and
+// that are still waiting there to be read (measured: the reducer of 2^18-slot tables 0.213 ->
+// 0.168 ms; non-temporal *stores* of the records cost the scatter more than they save here).
+template <bool kSplit>
+__device__ __forceinline__ BinRecord load_record_once(const BinTarget& bins, size_t first, uint32_t i) {
+    BinRecord rec;
+    if constexpr (kSplit) {
+        const RecordValues v = __builtin_nontemporal_load(static_cast<const RecordValues*>(bins.records) + first + i);
+        rec.slot_in_bin = __builtin_nontemporal_load(bins.slots + first + i);
+        rec.a0 = v.x;
+        rec.a1 = v.y;
+    } else {
+        const RecordWords w = __builtin_nontemporal_load(reinterpret_cast<const RecordWords*>(static_cast<const BinRecord*>(bins.records) + first + i));
+        const uint32_t w0 = w.x, w1 = w.y, w2 = w.z;  // copies first: a bit cast applied directly to a vector element reads element 0
+        rec.slot_in_bin = w0;
+        rec.a0 = __builtin_bit_cast(float, w1);
+        rec.a1 = __builtin_bit_cast(float, w2);
+    }
+    return rec;
 }
 
 // One level's slice of the table gradient as the scatter sees it: a pair of features per slot,
@@ -241,11 +300,7 @@ __device__ __forceinline__ bool append_record(State& c, const BinTarget& bins, u
     const uint32_t b = slot >> kBinSlotsLog2;
     const uint32_t pos = atomicAdd(&c.bin_count[b], 1u);
     if (pos >= bins.segment_capacity) return false;
-    BinRecord rec;
-    rec.slot_in_bin = slot & (kBinSlots - 1);
-    rec.a0 = a0;
-    rec.a1 = a1;
-    bins.records[(static_cast<size_t>(b) * bins.n_groups + group) * bins.segment_capacity + pos] = rec;
+    store_record(bins, (b * bins.n_groups + group) * bins.segment_capacity + pos, slot & (kBinSlots - 1), a0, a1);
     return true;
 }
 
@@ -310,7 +365,6 @@ __device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_gra
     uint32_t* const room = run_first + 64;                      // [bin] records the workgroup's segment can still take
     uint32_t* const header = room + 64;                         // [0] records staged, [1] whether every run fits
     uint4* const stage = reinterpret_cast<uint4*>(c.val);
-    char* const record_bytes = reinterpret_cast<char*>(bins.records);
     constexpr uint32_t kNoRoom = 0xFFFFFFFFu;
     constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
     static_for<kChunks>(PENC_BODY(chunk) {
@@ -376,11 +430,7 @@ __device__ __forceinline__ void stream_tile(State& c, const GradSlice& level_gra
             if (i < total) {
                 e = stage[i];
                 if (e.w != kNoRoom) {
-                    BinRecord rec;
-                    rec.slot_in_bin = e.x & (kBinSlots - 1);
-                    rec.a0 = __builtin_bit_cast(float, e.y);
-                    rec.a1 = __builtin_bit_cast(float, e.z);
-                    *reinterpret_cast<BinRecord*>(record_bytes + e.w * static_cast<uint32_t>(sizeof(BinRecord))) = rec;
+                    store_record(bins, e.w, e.x & (kBinSlots - 1), __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
                 } else {
                     spill = true;  // the segment is full: stage 3
                 }
@@ -417,7 +467,6 @@ __device__ __forceinline__ void stream_tile_many(State& c, const GradSlice& leve
     uint32_t* const dest = words + 2 * kMaxBins;         // [bin] index of the run's first record in the level's record array
     uint32_t* const wave_total = words + 3 * kMaxBins;   // [wave] records of the wave's 64 bins
     uint4* const stage = reinterpret_cast<uint4*>(c.val);
-    char* const record_bytes = reinterpret_cast<char*>(bins.records);
     constexpr uint32_t kNoRoom = 0xFFFFFFFFu;
     constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
     const uint32_t my_bin = threadIdx.x;  // the bin this thread looks after
@@ -482,11 +531,7 @@ __device__ __forceinline__ void stream_tile_many(State& c, const GradSlice& leve
             if (i < total) {
                 e = stage[i];
                 if (e.w != kNoRoom) {
-                    BinRecord rec;
-                    rec.slot_in_bin = e.x & (kBinSlots - 1);
-                    rec.a0 = __builtin_bit_cast(float, e.y);
-                    rec.a1 = __builtin_bit_cast(float, e.z);
-                    *reinterpret_cast<BinRecord*>(record_bytes + e.w * static_cast<uint32_t>(sizeof(BinRecord))) = rec;
+                    store_record(bins, e.w, e.x & (kBinSlots - 1), __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
                 } else {
                     spill = true;  // the segment is full: stage 3
                 }
@@ -529,7 +574,6 @@ __device__ __forceinline__ void stream_tile_wave(State& c, const GradSlice& leve
     uint32_t* start = count + 128;  // index of the run's first record in the level's record array
     uint32_t* room = count + 192;   // records the workgroup's segment of the bin can still take
     uint4* stage = reinterpret_cast<uint4*>(c.val) + wave * (kStageChunk * 64);
-    char* const record_bytes = reinterpret_cast<char*>(bins.records);
     constexpr uint32_t kNoRoom = 0xFFFFFFFFu;
     constexpr int kChunks = (D + 1 + kStageChunk - 1) / kStageChunk;
     static_for<kChunks>(PENC_BODY(chunk) {
@@ -573,11 +617,7 @@ __device__ __forceinline__ void stream_tile_wave(State& c, const GradSlice& leve
                 const uint32_t i = j * 64 + lane;
                 if (i < total) {
                     const uint4 e = stage[i];
-                    BinRecord rec;
-                    rec.slot_in_bin = e.x;
-                    rec.a0 = __builtin_bit_cast(float, e.y);
-                    rec.a1 = __builtin_bit_cast(float, e.z);
-                    *reinterpret_cast<BinRecord*>(record_bytes + e.w * static_cast<uint32_t>(sizeof(BinRecord))) = rec;
+                    store_record(bins, e.w, e.x, __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
                 }
             });
         } else {
@@ -605,11 +645,7 @@ __device__ __forceinline__ void stream_tile_wave(State& c, const GradSlice& leve
                 if (i < total) {
                     e = stage[i];
                     if (e.w != kNoRoom) {
-                        BinRecord rec;
-                        rec.slot_in_bin = e.x & (kBinSlots - 1);
-                        rec.a0 = __builtin_bit_cast(float, e.y);
-                        rec.a1 = __builtin_bit_cast(float, e.z);
-                        bins.records[e.w] = rec;
+                        store_record(bins, e.w, e.x & (kBinSlots - 1), __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
                     } else {
                         spill = true;  // the segment is full: stage 3
                     }
@@ -707,7 +743,7 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
     if (mode == kModeStream) {
         if (bins.n_bins > kStageBins) {
             stream_tile_many<D>(c, level_grad, bins, group, active, slot, a0, a1);
-        } else if constexpr (D <= 5) {  // measured: the workgroup-wide sort wins up to D = 5, the per-wave one from D = 6 on
+        } else if constexpr (D <= kWorkgroupSortMaxDim) {  // measured: the workgroup-wide sort wins up to D = 5, the per-wave one from D = 6 on
             stream_tile<D>(c, level_grad, bins, group, active, slot, a0, a1);
         } else {
             stream_tile_wave<D>(c, level_grad, bins, group, active, slot, a0, a1);
@@ -866,6 +902,7 @@ __device__ __forceinline__ void scatter_end(State& c, const GradSlice& level_gra
 // runs (the scattering kernel before it has completed, and bins do not overlap), so the final add is
 // a plain coalesced read-modify-write; workgroups that share a bin add with atomics (consecutive
 // addresses: one request per 64 bytes).
+template <bool kSplit>  // whether the records are split (the host knows: BinTarget::slots)
 __global__ void __launch_bounds__(kReduceBlock)
 bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity, uint32_t feat_pairs,
                   float* __restrict__ table_grad, int first_level) {
@@ -883,13 +920,13 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
     if (window[level] == 0.0f) return;  // masked level: its scattering workgroups wrote no counts
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     constexpr uint32_t kWaves = kReduceBlock / 64;
-    constexpr uint32_t kUnroll = 4;
+    constexpr uint32_t kUnroll = 4;  // even
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const uint32_t per_split = (bins.n_groups + gridDim.z - 1) / gridDim.z;
     const uint32_t group_begin = blockIdx.z * per_split;
     const uint32_t group_end = group_begin + per_split < bins.n_groups ? group_begin + per_split : bins.n_groups;
     const uint32_t* counts = bins.counts + static_cast<size_t>(bin) * bins.n_groups;
-    const BinRecord* recs = bins.records + static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;
+    const size_t first = static_cast<size_t>(bin) * bins.n_groups * bins.segment_capacity;  // the bin's first record
     // A bin nothing was appended to (the levels whose scattering workgroups summed in columns, a slot
     // range no point touches) ends here: the look at the counts overlaps the clearing of the sums,
     // and the barrier that follows the clearing carries the vote.
@@ -919,12 +956,12 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
             const auto fetch4 = [&](uint32_t step, BinRecord (&rec)[kShortUnroll]) {
                 const uint32_t k = 4 * step + quarter;  // < 64; lanes past the last segment hold a count of 0
                 const uint32_t count = static_cast<uint32_t>(__shfl(static_cast<int>(my_count), static_cast<int>(k)));
-                const BinRecord* seg = recs + static_cast<size_t>(g0 + k * kWaves) * bins.segment_capacity;
+                const uint32_t seg = (g0 + k * kWaves) * bins.segment_capacity;  // within the bin: below 2^29 like the level's records
 #pragma unroll
                 for (uint32_t u = 0; u < kShortUnroll; ++u) {
                     const uint32_t i = u * kShortLanes + l;
                     // (normal loads: neighbouring short segments share cache lines)
-                    rec[u] = *(i < count ? seg + i : recs);  // the bin's first record stands in where there is none
+                    rec[u] = load_record<kSplit>(bins, first, i < count ? seg + i : 0u);  // the bin's first record stands in where there is none
                 }
                 return count;
             };
@@ -946,38 +983,91 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
             continue;
         }
         const auto count_of = [&](uint32_t k) { return static_cast<uint32_t>(__builtin_amdgcn_readlane(my_count, k)); };
-        const auto fetch = [&](uint32_t k, uint32_t base, BinRecord (&rec)[kUnroll]) {
-            const uint32_t count = count_of(k);
-            const BinRecord* seg = recs + static_cast<size_t>(g0 + k * kWaves) * bins.segment_capacity;
+        // What a lane holds of one chunk, as loaded: split records are read two to a lane (16 bytes of
+        // values, 4 of slots: a quarter of the load instructions) and taken apart only when they are
+        // added, so that nothing between the loads and the previous chunk's adds waits for them.
+        typedef float ValuePair __attribute__((ext_vector_type(4)));
+        struct Loaded {
+            ValuePair values[kSplit ? kUnroll / 2 : 1];
+            uint32_t slots[kSplit ? kUnroll / 2 : 1];
+            RecordWords whole[kSplit ? 1 : kUnroll];
+        };
+        // record u of a lane's kUnroll is record index_of(base, u) of the segment
+        const auto index_of = [&](uint32_t base, uint32_t u) {
+            return kSplit ? base + ((u >> 1) * 64 + lane) * 2 + (u & 1) : base + u * 64 + lane;
+        };
+        struct Cursor {
+            uint32_t k, base;  // segment (of this wave's n_segments), first record of the chunk
+        };
+        const auto fetch = [&](const Cursor& at, Loaded& got) {
+            const uint32_t count = count_of(at.k);
+            const size_t seg = first + (g0 + at.k * kWaves) * bins.segment_capacity;
+            if constexpr (kSplit) {
+                const RecordValues* values = static_cast<const RecordValues*>(bins.records) + seg;  // 16-byte aligned:
+                const uint16_t* slots = bins.slots + seg;                                         // segments are multiples of four records
 #pragma unroll
-            for (uint32_t u = 0; u < kUnroll; ++u) {
-                const uint32_t i = base + u * 64 + lane;
-                rec[u] = load_record_once(seg + (i < count ? i : 0));
+                for (uint32_t u = 0; u < kUnroll; u += 2) {
+                    const uint32_t i = index_of(at.base, u);
+                    const uint32_t from = i < count ? i : 0u;  // even; an odd count's last pair reads one record of the segment's slack
+                    got.values[u / 2] = __builtin_nontemporal_load(reinterpret_cast<const ValuePair*>(values + from));
+                    got.slots[u / 2] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(slots + from));
+                }
+            } else {
+                const BinRecord* recs = static_cast<const BinRecord*>(bins.records) + seg;
+#pragma unroll
+                for (uint32_t u = 0; u < kUnroll; ++u) {
+                    const uint32_t i = index_of(at.base, u);
+                    got.whole[u] = __builtin_nontemporal_load(reinterpret_cast<const RecordWords*>(recs + (i < count ? i : 0u)));
+                }
             }
         };
-        uint32_t k = 0, base = 0;
-        while (k < n_segments && count_of(k) == 0u) ++k;
-        BinRecord cur[kUnroll], next[kUnroll];
-        if (k < n_segments) fetch(k, base, cur);
-        while (k < n_segments) {
-            const uint32_t count = count_of(k);
-            uint32_t next_k = k, next_base = base + kChunk;
-            if (next_base >= count) {
-                next_base = 0;
-                do ++next_k; while (next_k < n_segments && count_of(next_k) == 0u);
-            }
-            if (next_k < n_segments) fetch(next_k, next_base, next);
+        const auto add = [&](const Cursor& at, const Loaded& got) {
+            const uint32_t count = count_of(at.k);
 #pragma unroll
-            for (uint32_t u = 0; u < kUnroll; ++u)
-                if (base + u * 64 + lane < count) {
-                    const uint32_t cell = cur[u].slot_in_bin;
-                    __hip_atomic_fetch_add(&acc0[cell], static_cast<double>(cur[u].a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                    __hip_atomic_fetch_add(&acc1[cell], static_cast<double>(cur[u].a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            for (uint32_t u = 0; u < kUnroll; ++u) {
+                uint32_t cell;
+                float a0, a1;
+                if constexpr (kSplit) {
+                    const ValuePair v = got.values[u / 2];
+                    const float v0 = v.x, v1 = v.y, v2 = v.z, v3 = v.w;  // copies first: a bit cast applied directly to a vector element reads element 0
+                    cell = (u & 1) ? got.slots[u / 2] >> 16 : got.slots[u / 2] & 0xFFFFu;
+                    a0 = (u & 1) ? v2 : v0;
+                    a1 = (u & 1) ? v3 : v1;
+                } else {
+                    const RecordWords w = got.whole[u];
+                    const uint32_t w0 = w.x, w1 = w.y, w2 = w.z;
+                    cell = w0;
+                    a0 = __builtin_bit_cast(float, w1);
+                    a1 = __builtin_bit_cast(float, w2);
                 }
-#pragma unroll
-            for (uint32_t u = 0; u < kUnroll; ++u) cur[u] = next[u];
-            k = next_k;
-            base = next_base;
+                if (index_of(at.base, u) < count) {
+                    __hip_atomic_fetch_add(&acc0[cell], static_cast<double>(a0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                    __hip_atomic_fetch_add(&acc1[cell], static_cast<double>(a1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                }
+            }
+        };
+        // the chunk after `at`: the next kChunk records of its segment, or the start of the next segment that has any
+        const auto after = [&](Cursor at) {
+            at.base += kChunk;
+            if (at.base >= count_of(at.k)) {
+                at.base = 0;
+                do ++at.k; while (at.k < n_segments && count_of(at.k) == 0u);
+            }
+            return at;
+        };
+        // two sets of registers take turns, so a chunk's loads stay in flight over the other chunk's adds
+        Cursor a{0u, 0u};
+        while (a.k < n_segments && count_of(a.k) == 0u) ++a.k;
+        Loaded got_a, got_b;
+        if (a.k < n_segments) fetch(a, got_a);
+        while (a.k < n_segments) {
+            const Cursor b = after(a);
+            if (b.k < n_segments) fetch(b, got_b);
+            add(a, got_a);
+            if (b.k >= n_segments) break;
+            a = after(b);
+            if (a.k < n_segments) fetch(a, got_a);
+            add(b, got_b);
         }
     }
     __syncthreads();
