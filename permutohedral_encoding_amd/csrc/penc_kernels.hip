@@ -201,7 +201,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     scatter_begin(state);
     const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair_level % feat_pairs) * 2,
-                               2 * feat_pairs};
+                               2 * feat_pairs, bins.records != nullptr ? bins.direct : nullptr};
     // Everything a thread reads lies within its group of at most 16 x 512 points, so the addresses are
     // wave-uniform 64-bit bases (scalar registers) plus 32-bit per-thread offsets.
     const uint32_t last_in_group = static_cast<uint32_t>(n_points - 1 - group_base);
@@ -513,10 +513,11 @@ transpose_kernel(const float* __restrict__ src, int64_t src_row_stride, float* _
         for (int col = wave; col < cols; col += kBlock / 64) dst[static_cast<int64_t>(col) * rows + row0 + lane] = tile[lane * stride + col];
 }
 
-__global__ void __launch_bounds__(kBlock) fill_zero_kernel(float2* __restrict__ p, size_t n2) {
-    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
-    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n2; i += stride)
-        p[i] = make_float2(0.0f, 0.0f);
+// Clears two arrays (the second may be empty): n2 and m2 count 8-byte units.
+__global__ void __launch_bounds__(kBlock) fill_zero_kernel(float2* __restrict__ p, size_t n2, float2* __restrict__ q, size_t m2) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock, first = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
+    for (size_t i = first; i < n2; i += stride) p[i] = make_float2(0.0f, 0.0f);
+    for (size_t i = first; i < m2; i += stride) q[i] = make_float2(0.0f, 0.0f);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -561,14 +562,16 @@ inline bool table_aligned(const TableRef& t, int nr_feat) {
     return (reinterpret_cast<uintptr_t>(t.values) & ((slot_bytes < 16u ? slot_bytes : 16u) - 1u)) == 0;
 }
 
-// Clears the table gradient with a fill kernel (float2 granularity: the array is only guaranteed
-// 8-byte alignment).  A kernel rather than hipMemsetAsync so that callers may capture the call in
-// a HIP graph.
-inline int clear_table_grad(float* g, int pair_levels, int capacity, hipStream_t st) {
+// Clears the table gradient, and the bins' `direct` flags when there are bins (`flags` of
+// `flag_bytes`, a multiple of 8), with a fill kernel (float2 granularity: the gradient is only
+// guaranteed 8-byte alignment).  A kernel rather than hipMemsetAsync so that callers may capture
+// the call in a HIP graph.
+inline int clear_table_grad(float* g, int pair_levels, int capacity, void* flags, size_t flag_bytes, hipStream_t st) {
     const size_t n2 = static_cast<size_t>(pair_levels) * capacity;
     const size_t want = (n2 + kBlock * 8 - 1) / (kBlock * 8);
     const unsigned blocks = static_cast<unsigned>(want < 8192 ? want : 8192);
-    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(kBlock), 0, st, reinterpret_cast<float2*>(g), n2);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(kBlock), 0, st, reinterpret_cast<float2*>(g), n2,
+                       static_cast<float2*>(flags), flags != nullptr ? flag_bytes / sizeof(float2) : size_t{0});
     return check_launch();
 }
 
@@ -579,8 +582,14 @@ inline int clear_table_grad(float* g, int pair_levels, int capacity, hipStream_t
 struct BinPlan {
     bool enabled = false;
     int levels_per_pass = 0;
-    BinTarget target{};
+    BinTarget target{};       // of the first pass; target.direct covers all levels, a pass starts at its first level's flags
+    size_t direct_bytes = 0;  // size of target.direct (to be cleared with the gradient)
 };
+
+// Bytes of the `direct` flags of all levels (one 4-byte flag per level and bin), padded to the workspace's alignment.
+inline size_t direct_flag_bytes(int levels, uint32_t n_bins) {
+    return (static_cast<size_t>(levels) * n_bins * sizeof(uint32_t) + 255u) & ~size_t{255};
+}
 
 inline uint32_t bins_for_capacity(int capacity) {
     return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
@@ -635,8 +644,9 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int t
     if (n * (pos_dim + 1) * kMinSlotsPerContribution <= capacity) return p;
     const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
     const size_t lost = base - reinterpret_cast<uintptr_t>(workspace);
-    if (bytes < lost + 4096) return p;
-    bytes -= lost + 256;
+    const size_t flag_bytes = direct_flag_bytes(levels, n_bins);
+    if (bytes < lost + flag_bytes + 4096) return p;
+    bytes -= lost + flag_bytes + 256;
     const size_t segments = static_cast<size_t>(n_bins) * n_groups;
     const bool split = record_bytes(pos_dim, n_bins) == kSplitRecordBytes;
     uint32_t cap = wanted_segment_capacity(pos_dim, n_bins, tiles_per_group);
@@ -657,11 +667,14 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int t
     p.target.n_bins = n_bins;
     p.target.n_groups = n_groups;
     p.target.segment_capacity = cap;
-    p.target.counts = reinterpret_cast<uint32_t*>(base);
+    p.target.direct = reinterpret_cast<uint32_t*>(base);
+    p.direct_bytes = flag_bytes;
+    const uintptr_t counts_at = base + flag_bytes;
+    p.target.counts = reinterpret_cast<uint32_t*>(counts_at);
     const size_t counts_bytes = (static_cast<size_t>(p.levels_per_pass) * segments * sizeof(uint32_t) + 255u) & ~size_t{255};
     const size_t records_per_pass = static_cast<size_t>(p.levels_per_pass) * segments * cap;
-    p.target.records = reinterpret_cast<void*>(base + counts_bytes);
-    p.target.slots = split ? reinterpret_cast<uint16_t*>(base + counts_bytes + records_per_pass * sizeof(RecordValues)) : nullptr;
+    p.target.records = reinterpret_cast<void*>(counts_at + counts_bytes);
+    p.target.slots = split ? reinterpret_cast<uint16_t*>(counts_at + counts_bytes + records_per_pass * sizeof(RecordValues)) : nullptr;
     p.enabled = true;
     return p;
 }
@@ -678,6 +691,18 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
     unsigned splits = pairs >= kReduceWorkgroupsWanted ? 1u : (kReduceWorkgroupsWanted + pairs - 1) / pairs;
     if (splits > p.target.n_groups) splits = p.target.n_groups;
     if (splits > kMaxReduceSplits) splits = kMaxReduceSplits;
+    // many bins with a few thousand records each: workgroups that keep their bin and walk several levels
+    if (p.target.slots == nullptr && p.target.n_bins > static_cast<uint32_t>(kStageBins) && splits == 1 &&
+        p.target.segment_capacity <= kLevelsMaxSegment && p.target.n_groups <= static_cast<uint32_t>(kReduceBlock)) {
+        const unsigned levels = static_cast<unsigned>(n_levels_in_pass);
+        unsigned per_bin = (levels + kLevelsMaxPerWorkgroup - 1) / kLevelsMaxPerWorkgroup;
+        const unsigned to_fill = (2 * kReduceWorkgroupsWanted + p.target.n_bins - 1) / p.target.n_bins;  // four workgroups per compute unit, one after the other
+        if (per_bin < to_fill) per_bin = to_fill;
+        if (per_bin > levels) per_bin = levels;
+        hipLaunchKernelGGL(bin_reduce_levels_kernel, dim3(p.target.n_bins, per_bin), dim3(kReduceBlock), 0, st, p.target, window,
+                           static_cast<uint32_t>(capacity), feat_pairs, table_grad, first_level, static_cast<uint32_t>(levels));
+        return check_launch();
+    }
     const dim3 grid(p.target.n_bins, n_levels_in_pass, splits);
     if (p.target.slots != nullptr)
         hipLaunchKernelGGL(bin_reduce_kernel<true>, grid, dim3(kReduceBlock), 0, st, p.target, window,
@@ -786,15 +811,19 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
     // every pair of features is scattered like a level of its own (see backward_table_kernel)
     const uint32_t feat_pairs = static_cast<uint32_t>(nr_feat / 2);
     const int pair_levels = nr_levels * static_cast<int>(feat_pairs);
-    if (int rc = clear_table_grad(lattice_values_grad, pair_levels, capacity, st)) return rc;
     const int tiles_per_group = table_backward_tiles(nr_positions, pair_levels);
-    const BinPlan plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
+    BinPlan plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
+    if (int rc = clear_table_grad(lattice_values_grad, pair_levels, capacity, plan.enabled ? plan.target.direct : nullptr,
+                                  plan.direct_bytes, st))
+        return rc;
+    uint32_t* const direct_flags = plan.target.direct;
     const int per_pass = plan.enabled ? plan.levels_per_pass : pair_levels;
     const uint32_t dies = dies_of_current_device();
     for (int first = 0; first < pair_levels; first += per_pass) {
         const int count = pair_levels - first < per_pass ? pair_levels - first : per_pass;
         const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + dies - 1) / dies * dies;
         const dim3 grid(padded_groups * static_cast<unsigned>(count));
+        if (plan.enabled) plan.target.direct = direct_flags + static_cast<size_t>(first) * plan.target.n_bins;
 #define PENC_LAUNCH_TABLE(ROW_MAJOR, SECOND_ORDER)                                                                         \
     PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER>), grid,                  \
                                                 dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
@@ -941,7 +970,7 @@ size_t penc_scatter_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_le
                                                 wanted_segment_capacity(pos_dim, n_bins, tiles));
         per_level = need > per_level ? need : per_level;
     }
-    return per_level * static_cast<size_t>(levels_per_pass) + 1024;
+    return per_level * static_cast<size_t>(levels_per_pass) + direct_flag_bytes(nr_levels, n_bins) + 1024;
 }
 
 size_t penc_positions_workspace_bytes(int pos_dim, int64_t nr_positions, int nr_levels) {

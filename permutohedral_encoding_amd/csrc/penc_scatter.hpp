@@ -93,11 +93,14 @@ constexpr size_t kSplitRecordBytes = sizeof(RecordValues) + sizeof(uint16_t);
 //   records [level_in_pass][bin][group][segment_capacity]   12-byte records, or the 8-byte values of split ones
 //   slots   [level_in_pass][bin][group][segment_capacity]   the 2-byte slots of split records; nullptr otherwise
 //   counts  [level_in_pass][bin][group]            records actually written (<= segment_capacity)
+//   direct  [level_in_pass][bin]                   nonzero once anything has been added straight into the gradient
+//                                                  in the bin's slot range (cleared with the gradient; see GradSlice)
 // `records` == nullptr disables binning.
 struct BinTarget {
     void* records;
     uint16_t* slots;
     uint32_t* counts;
+    uint32_t* direct;
     uint32_t n_bins;
     uint32_t n_groups;
     uint32_t segment_capacity;
@@ -112,6 +115,7 @@ __device__ __forceinline__ BinTarget bins_of_level(const BinTarget& pass, uint32
         t.records = static_cast<char*>(pass.records) + records * (pass.slots != nullptr ? sizeof(RecordValues) : sizeof(BinRecord));
         if (pass.slots != nullptr) t.slots += records;
         t.counts += segments;
+        t.direct += static_cast<size_t>(k) * pass.n_bins;
     }
     return t;
 }
@@ -174,10 +178,19 @@ __device__ __forceinline__ BinRecord load_record_once(const BinTarget& bins, siz
 // One level's slice of the table gradient as the scatter sees it: a pair of features per slot,
 // `slot_floats` floats from one slot to the next (2 when a level has two features; with four, the
 // slice of features (0,1) or (2,3) of an array whose slots are four floats apart).
+// `direct` (the level's BinTarget::direct, or nullptr without bins) is told about every add that goes
+// straight into the gradient: a bin whose slot range received none still holds the zeros it was
+// cleared to when its reducer workgroup arrives, which can then store its sums without reading
+// the gradient first (on a 2^22-slot table, whose gradient no cache holds, that read is a third
+// of the reducer's traffic).
 struct GradSlice {
     float* base;
     uint32_t slot_floats;
+    uint32_t* direct;
     __device__ __forceinline__ float* at(uint32_t slot) const { return base + static_cast<size_t>(slot) * slot_floats; }
+    __device__ __forceinline__ void mark_direct(uint32_t slot) const {
+        if (direct != nullptr) direct[slot >> kBinSlotsLog2] = 1u;
+    }
 };
 
 __device__ __forceinline__ void global_add(float* addr, float v) {
@@ -235,6 +248,7 @@ __device__ __forceinline__ void global_add_pairs(const GradSlice& level_grad, bo
                                                  float a0, float a1) {
     constexpr int kFromEven = 0xA0;  // quad_perm:[0,0,2,2]
     constexpr int kFromOdd = 0xF5;   // quad_perm:[1,1,3,3]
+    if (need) level_grad.mark_direct(slot);
     const int odd = threadIdx.x & 1;
     const int slot_i = static_cast<int>(slot), need_i = need ? 1 : 0;
     const int a0_i = __builtin_bit_cast(int, a0), a1_i = __builtin_bit_cast(int, a1);
@@ -725,6 +739,7 @@ __device__ __forceinline__ void column_flush(State& c, const GradSlice& level_gr
             // straight into the gradient: a level in column mode leaves a few dozen sums per workgroup, and
             // as records they would only make every bin's reducer workgroup run for a handful of them
             float* g = level_grad.at(static_cast<uint32_t>(owner));
+            level_grad.mark_direct(static_cast<uint32_t>(owner));
             global_add(g, static_cast<float>(s0));
             global_add(g + 1, static_cast<float>(s1));
         }
@@ -825,6 +840,7 @@ __device__ __forceinline__ void cache_flush(State& c, const GradSlice& level_gra
             const bool binned = bins.records != nullptr && append_record(c, bins, group, static_cast<uint32_t>(owner), v0, v1);
             if (!binned) {
                 float* g = level_grad.at(static_cast<uint32_t>(owner));
+                level_grad.mark_direct(static_cast<uint32_t>(owner));
                 global_add(g, v0);
                 global_add(g + 1, v1);
             }
@@ -1071,10 +1087,12 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
         }
     }
     __syncthreads();
-    const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs};
+    const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr};
     const uint32_t slot0 = bin << kBinSlotsLog2;
     const bool alone = gridDim.z == 1;
     if (alone) {
+        // nothing but this workgroup has added to the bin's slots since the gradient was cleared: the sums are the result
+        const bool untouched_so_far = bins.direct[bin] == 0u;
         // all of a thread's read-modify-writes at once: the loads are issued together, not one per trip
         constexpr int kMine = kBinSlots / kReduceBlock;
         float2 sum[kMine], g[kMine];
@@ -1089,7 +1107,8 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
 #pragma unroll
         for (int k = 0; k < kMine; ++k) {
             const uint32_t s = static_cast<uint32_t>(k) * kReduceBlock + threadIdx.x;
-            if (touched[k]) g[k] = *reinterpret_cast<const float2*>(level_grad.at(slot0 + s));
+            g[k] = make_float2(0.0f, 0.0f);
+            if (touched[k] && !untouched_so_far) g[k] = *reinterpret_cast<const float2*>(level_grad.at(slot0 + s));
         }
 #pragma unroll
         for (int k = 0; k < kMine; ++k) {
@@ -1109,6 +1128,159 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
             global_add(&cell->x, static_cast<float>(v0));
             global_add(&cell->y, static_cast<float>(v1));
         }
+    }
+}
+
+// The reducer of tables with hundreds of bins.  There a scattering workgroup leaves only a few
+// dozen records in each of its segments and a (bin, level) has a few thousand in all, so a workgroup of
+// bin_reduce_kernel is a chain of latencies (launch, counts, records, gradient) with nothing to overlap
+// them: its 128 KiB of sums allow one workgroup per compute unit.  Here a workgroup keeps its bin and walks
+// several levels (blockIdx.y, + gridDim.y, ...): the counts of all its levels are fetched at once
+// (levels that left no records cost nothing more), and over the sequence of (level, 64 segments)
+// steps that remain the counts are fetched two steps and the records one step ahead of the adds, so the
+// loads of the next level are in flight while this level's sums are added and written out.
+// A quarter of a wave reads a segment, kLevelsShortUnroll records per lane: needs segments of at
+// most kLevelsMaxSegment records, whole (12-byte) records, at most kReduceBlock groups and
+// at most kLevelsMaxPerWorkgroup levels per workgroup (the host checks all four).
+constexpr uint32_t kLevelsShortLanes = 16, kLevelsShortUnroll = 8;
+constexpr uint32_t kLevelsMaxSegment = kLevelsShortLanes * kLevelsShortUnroll;
+constexpr uint32_t kLevelsMaxPerWorkgroup = 12;
+__global__ void __launch_bounds__(kReduceBlock)
+bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_t capacity, uint32_t feat_pairs,
+                         float* __restrict__ table_grad, int first_level, uint32_t n_levels_in_pass) {
+    __shared__ double acc0[kBinSlots];
+    __shared__ double acc1[kBinSlots];
+    __shared__ uint32_t masks[2];  // bit i: the workgroup's i-th level [0] has records in this bin, [1] got direct adds in this bin's slots
+    const uint32_t bin = blockIdx.x, my_first = blockIdx.y, my_stride = gridDim.y;
+    const uint32_t n_mine = (n_levels_in_pass - my_first + my_stride - 1) / my_stride;  // blockIdx.y < n_levels_in_pass
+    const uint32_t n_bins = pass_bins.n_bins, n_groups = pass_bins.n_groups, seg_cap = pass_bins.segment_capacity;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the workgroup's i-th level within the pass, and where its segments of this bin start (counted in segments)
+    const auto level_in_pass = [&](uint32_t i) { return my_first + i * my_stride; };
+    const auto first_segment = [&](uint32_t i) { return (static_cast<size_t>(level_in_pass(i)) * n_bins + bin) * n_groups; };
+    if (threadIdx.x < 2) masks[threadIdx.x] = 0u;
+    for (int s = threadIdx.x; s < kBinSlots; s += kReduceBlock) {
+        acc0[s] = 0.0;
+        acc1[s] = 0.0;
+    }
+    // which of the levels have records here (thread g looks at group g's count of every level, all loads at once)
+    uint32_t seen[kLevelsMaxPerWorkgroup];
+#pragma unroll
+    for (uint32_t i = 0; i < kLevelsMaxPerWorkgroup; ++i) {
+        seen[i] = 0u;
+        if (i < n_mine) {
+            const uint32_t pair_level = static_cast<uint32_t>(first_level) + level_in_pass(i);
+            // (a masked level's scattering workgroups wrote no counts)
+            if (window[pair_level / feat_pairs] != 0.0f && threadIdx.x < n_groups) seen[i] = pass_bins.counts[first_segment(i) + threadIdx.x];
+        }
+    }
+    uint32_t direct = 0u;
+    if (threadIdx.x < n_mine) direct = pass_bins.direct[static_cast<size_t>(level_in_pass(threadIdx.x)) * n_bins + bin];
+    __syncthreads();  // the masks are cleared
+    uint32_t found = 0u;
+#pragma unroll
+    for (uint32_t i = 0; i < kLevelsMaxPerWorkgroup; ++i)
+        if (__ballot(seen[i] != 0u) != 0ull) found |= 1u << i;
+    if (lane == 0 && found != 0u) atomicOr(&masks[0], found);
+    if (direct != 0u) atomicOr(&masks[1], 1u << threadIdx.x);
+    __syncthreads();
+    const uint32_t todo = masks[0], direct_mask = masks[1];
+    if (todo == 0u) return;
+
+    // a step: 64 segments of one level, one per quarter wave
+    constexpr uint32_t kEnd = 32;
+    struct Cursor {
+        uint32_t i, step;  // the workgroup's i-th level (kEnd: past the last), segments 64 * step ...
+    };
+    const uint32_t n_steps = (n_groups + 63) / 64;
+    const auto after = [&](Cursor at) {
+        if (++at.step < n_steps) return at;
+        const uint32_t rest = at.i + 1 < 32 ? todo >> (at.i + 1) : 0u;
+        return Cursor{rest != 0u ? at.i + 1 + static_cast<uint32_t>(__builtin_ctz(rest)) : kEnd, 0u};
+    };
+    const uint32_t reader = wave * 4 + lane / kLevelsShortLanes, l = lane % kLevelsShortLanes;
+    const auto load_count = [&](const Cursor& at) {
+        const uint32_t g = at.step * 64 + reader;
+        return g < n_groups ? pass_bins.counts[first_segment(at.i) + g] : 0u;
+    };
+    struct Loaded {
+        RecordWords rec[kLevelsShortUnroll];
+        uint32_t count;
+    };
+    const BinRecord* const records = static_cast<const BinRecord*>(pass_bins.records);
+    const auto fetch = [&](const Cursor& at, uint32_t count, Loaded& got) {
+        const uint32_t g = at.step * 64 + reader;
+        const BinRecord* seg = records + (first_segment(at.i) + (g < n_groups ? g : 0u)) * seg_cap;
+        got.count = count;
+#pragma unroll
+        for (uint32_t u = 0; u < kLevelsShortUnroll; ++u) {
+            const uint32_t idx = u * kLevelsShortLanes + l;
+            // (normal loads: neighbouring short segments share cache lines); the pass's first record stands in where there is none
+            got.rec[u] = *reinterpret_cast<const RecordWords*>(idx < count ? seg + idx : records);
+        }
+    };
+    const auto add = [&](const Loaded& got) {
+#pragma unroll
+        for (uint32_t u = 0; u < kLevelsShortUnroll; ++u) {
+            const RecordWords w = got.rec[u];
+            const uint32_t w0 = w.x, w1 = w.y, w2 = w.z;  // copies first: a bit cast applied directly to a vector element reads element 0
+            if (u * kLevelsShortLanes + l < got.count) {
+                __hip_atomic_fetch_add(&acc0[w0], static_cast<double>(__builtin_bit_cast(float, w1)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&acc1[w0], static_cast<double>(__builtin_bit_cast(float, w2)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+    };
+    // Adds the sums of the workgroup's i-th level into the gradient and clears them.  Nothing else touches
+    // the bin's slots of that level while this kernel runs, so the add is a plain read-modify-write, or a
+    // store where nothing was added since the gradient was cleared.
+    const auto flush = [&](uint32_t i) {
+        __syncthreads();
+        const uint32_t pair_level = static_cast<uint32_t>(first_level) + level_in_pass(i);
+        const uint32_t level = pair_level / feat_pairs, pair = pair_level % feat_pairs;
+        const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr};
+        const uint32_t slot0 = bin << kBinSlotsLog2;
+        const bool untouched_so_far = ((direct_mask >> i) & 1u) == 0u;
+        constexpr int kMine = kBinSlots / kReduceBlock;
+#pragma unroll
+        for (int k = 0; k < kMine; ++k) {
+            const uint32_t s = static_cast<uint32_t>(k) * kReduceBlock + threadIdx.x;
+            const double v0 = acc0[s], v1 = acc1[s];
+            if (v0 != 0.0 || v1 != 0.0) {
+                acc0[s] = 0.0;
+                acc1[s] = 0.0;
+                if (slot0 + s < capacity) {
+                    float2* cell = reinterpret_cast<float2*>(level_grad.at(slot0 + s));
+                    float2 g = make_float2(0.0f, 0.0f);
+                    if (!untouched_so_far) g = *cell;
+                    g.x += static_cast<float>(v0);
+                    g.y += static_cast<float>(v1);
+                    *cell = g;
+                }
+            }
+        }
+        __syncthreads();
+    };
+    // two sets of registers take turns for the records, two registers for the counts
+    Cursor it0{static_cast<uint32_t>(__builtin_ctz(todo)), 0u};
+    Cursor it1 = after(it0);
+    uint32_t count_x = load_count(it0), count_y = it1.i != kEnd ? load_count(it1) : 0u;
+    Loaded got_a, got_b;
+    fetch(it0, count_x, got_a);
+    while (true) {
+        const Cursor it2 = it1.i != kEnd ? after(it1) : it1;
+        if (it2.i != kEnd) count_x = load_count(it2);
+        if (it1.i != kEnd) fetch(it1, count_y, got_b);
+        add(got_a);
+        if (it1.i != it0.i) flush(it0.i);
+        if (it1.i == kEnd) break;
+        const Cursor it3 = it2.i != kEnd ? after(it2) : it2;
+        if (it3.i != kEnd) count_y = load_count(it3);
+        if (it2.i != kEnd) fetch(it2, count_x, got_a);
+        add(got_b);
+        if (it2.i != it1.i) flush(it1.i);
+        if (it2.i == kEnd) break;
+        it0 = it2;
+        it1 = it3;
     }
 }
 
