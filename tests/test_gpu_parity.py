@@ -741,6 +741,29 @@ def test_segments_overflow_with_more_bins_than_lanes():
     _table_gradients_match(p, d, cap, "segments overflow, 128 bins")
 
 
+@pytest.mark.parametrize("feat,cap,levels,n", [(4, 1 << 21, 13, 90000), (2, (1 << 21) + 1, 7, 90000), (2, 1 << 22, 16, 140000)])
+def test_many_bins_levels_shared_by_a_reducer_workgroup(feat, cap, levels, n):
+    """Tables with hundreds of slot ranges, whose segments hold a few dozen records, are reduced by
+    workgroups that keep their range and walk several levels: level lists that divide unevenly among
+    them (26 pairs of features over 4 workgroups, 7 levels over 4, 16 over 2), masked levels in
+    between, coarse levels whose scattering workgroups add straight into the gradient (so the
+    reducer must add to what is there), and one slot range past a power of two.  First- and
+    second-order table gradients against the oracle."""
+    d = 3
+    p = random_problem(d, n, levels, cap, seed=300 + levels, sigma_range=(1.0, 2e-3), nr_feat=feat)
+    p["window"][[1, levels - 2]] = 0.0
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
+    inp = gpu_input(p, need_pos_grad=False)
+    tg, _ = enc.backward(inp, to_gpu(p["grad"]))
+    want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
+    assert not tg[1].any() and not tg[levels - 2].any()
+    tg2, _ = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "second-order table gradient")
+
+
 def test_records_crowd_one_bin():
     """Points chosen so that, at the finest level, at least three of their four vertices fall into the
     first of four slot ranges: the tile's records are all distinct (the workgroup streams them sorted
