@@ -338,10 +338,12 @@ def main():
     phase_bytes = {"forward": ab["forward"]}
     phase_bytes["backward"] = (ab["backward_table"] if want_table else 0.0) + (ab["backward_pos"] if want_pos else 0.0)
     phase_bytes["double_backward"] = ab["double_backward"]
+    # tables with more than 64 slot ranges of 8192 slots are reduced by workgroups that walk several levels
+    reducer = "bin_reduce_levels_kernel" if w.capacity > 64 * 8192 else "bin_reduce_kernel"
     kernel_names = {"forward": "forward_kernel",
-                    "backward": "+".join((["fill_zero_kernel", "backward_table_kernel", "bin_reduce_kernel"] if want_table else [])
+                    "backward": "+".join((["fill_zero_kernel", "backward_table_kernel", reducer] if want_table else [])
                                          + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else [])),
-                    "double_backward": "grad_grad_kernel+fill_zero_kernel+backward_table_kernel<second order>+bin_reduce_kernel"}
+                    "double_backward": "grad_grad_kernel+fill_zero_kernel+backward_table_kernel<second order>+" + reducer}
     dominant = max(phase_ms, key=phase_ms.get)
     achieved = phase_bytes[dominant] * w.point_levels / (phase_ms[dominant] * 1e-3) / 1e9
     # HBM bytes per launch and vector instructions per point-level come from the committed counter

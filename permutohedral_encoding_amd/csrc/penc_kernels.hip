@@ -100,9 +100,10 @@ __device__ __forceinline__ Vertices<D, F> load_vertices(const T* __restrict__ le
 // ------------------------------------------------------------------------------------------
 // forward (EncodingGPU.cuh:68-256)
 //
-// Measured alternatives to one thread per (point, level), all slower or equal: 2 or 4 points per
+// One thread per point and one or two levels (the host says which).  Measured alternatives, all
+// slower or equal: 2 or 4 points per
 // thread (more loads in flight per lane: no gain, the kernel already runs at the rate this GPU
-// sustains for random 8-byte loads from a 2 MiB slice); walking the levels inside the thread with
+// sustains for random 8-byte loads from a 2 MiB slice); walking all the levels inside the thread with
 // the positions kept in registers (20% slower at 2^20 points, 3x slower at 2^16: fewer, longer
 // waves lose more than the re-read positions cost); interleaving workgroups of a coarse
 // (compute-bound) and a fine (gather-bound) level, which takes the fine level's slice out of L2
@@ -110,51 +111,58 @@ __device__ __forceinline__ Vertices<D, F> load_vertices(const T* __restrict__ le
 
 template <int D, int F, typename T>
 __global__ void __launch_bounds__(kBlock)
-forward_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
+forward_kernel(int n_points, int n_levels, int n_all_levels, int levels_per_thread, uint32_t capacity, uint32_t cap_mask,
                const float* __restrict__ positions, const T* __restrict__ table,
                const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                const float* __restrict__ window, float* __restrict__ sliced, float points_scaling) {
     const int n = blockIdx.x * kBlock + threadIdx.x;
     if (n >= n_points) return;
-    const int level = blockIdx.y;
-    float* out = sliced + (static_cast<size_t>(level) * F) * n_points + n;  // feature k at out[k * n_points]
+    __shared__ uint2 columns[(D + 1) * kBlock];
+    const fvec<D> point = load_point<D>(positions, n);
+    // The levels of a thread are `gridDim.y` apart: with the usual coarse-to-fine level list a thread that
+    // takes two pairs a level whose gathers hit the first-level cache with one that waits for the L2.
+#pragma unroll 1
+    for (int k2 = 0; k2 < levels_per_thread; ++k2) {
+        const int level = static_cast<int>(blockIdx.y) + k2 * static_cast<int>(gridDim.y);
+        if (level >= n_all_levels) break;
+        float* out = sliced + (static_cast<size_t>(level) * F) * n_points + n;  // feature k at out[k * n_points]
 
-    if (level >= n_levels) {  // extra levels carrying the raw positions (:106-121)
-        const int src = (level - n_levels) * F;
-        const float* p = positions + static_cast<size_t>(n) * D;
+        if (level >= n_levels) {  // extra levels carrying the raw positions (:106-121)
+            const int src = (level - n_levels) * F;
+            const float* p = positions + static_cast<size_t>(n) * D;
+            static_for<F>(PENC_BODY(k) {
+                PENC_INDEX(k);
+                out[static_cast<size_t>(k) * n_points] = src + k < D ? p[src + k] * points_scaling : 0.0f;
+            });
+            continue;
+        }
+        const float w_level = window[level];
+        if (w_level == 0.0f) {
+            static_for<F>(PENC_BODY(k) {
+                PENC_INDEX(k); out[static_cast<size_t>(k) * n_points] = 0.0f; });
+            continue;
+        }
+        const Located<D> s = locate<D>(point, random_shift + level * D, scale_factor + level * D);
+        // residuals and hash steps into rank order through LDS: up to 6% faster than the select chains
+        // of vertex_hashes() / barycentric() at D = 8, equal at D = 3
+        uvec<D + 1> h;
+        fvec<D + 1> sorted;
+        sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, s.delta, s.hash0, sorted, h);
+        const fvec<D + 1> w = barycentric_of_sorted<D>(sorted);
+        const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+        fvec<F> acc = 0.0f;
+        static_for<D + 1>(PENC_BODY(r) {
+            PENC_INDEX(r);
+            const float wr = w[r] * w_level;
+            static_for<F>(PENC_BODY(k) {
+                PENC_INDEX(k); acc[k] = acc[k] + v.f[k][r] * wr; });
+        });
         static_for<F>(PENC_BODY(k) {
             PENC_INDEX(k);
-            out[static_cast<size_t>(k) * n_points] = src + k < D ? p[src + k] * points_scaling : 0.0f;
+            // written once and not read here: the non-temporal hint keeps it from displacing the level's table slice
+            __builtin_nontemporal_store(acc[k], out + static_cast<size_t>(k) * n_points);
         });
-        return;
     }
-    const float w_level = window[level];
-    if (w_level == 0.0f) {
-        static_for<F>(PENC_BODY(k) {
-            PENC_INDEX(k); out[static_cast<size_t>(k) * n_points] = 0.0f; });
-        return;
-    }
-    const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, scale_factor + level * D);
-    // residuals and hash steps into rank order through LDS: up to 6% faster than the select chains
-    // of vertex_hashes() / barycentric() at D = 8, equal at D = 3
-    __shared__ uint2 columns[(D + 1) * kBlock];
-    uvec<D + 1> h;
-    fvec<D + 1> sorted;
-    sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, s.delta, s.hash0, sorted, h);
-    const fvec<D + 1> w = barycentric_of_sorted<D>(sorted);
-    const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
-    fvec<F> acc = 0.0f;
-    static_for<D + 1>(PENC_BODY(r) {
-        PENC_INDEX(r);
-        const float wr = w[r] * w_level;
-        static_for<F>(PENC_BODY(k) {
-            PENC_INDEX(k); acc[k] = acc[k] + v.f[k][r] * wr; });
-    });
-    static_for<F>(PENC_BODY(k) {
-        PENC_INDEX(k);
-        // written once and not read here: the non-temporal hint keeps it from displacing the level's table slice
-        __builtin_nontemporal_store(acc[k], out + static_cast<size_t>(k) * n_points);
-    });
 }
 
 // ------------------------------------------------------------------------------------------
@@ -355,41 +363,46 @@ reduce_level_groups_kernel(const float* __restrict__ partial, int n_groups, size
 
 template <int D, int F, typename T>
 __global__ void __launch_bounds__(kBlock)
-grad_grad_kernel(int n_points, int n_levels, uint32_t capacity, uint32_t cap_mask,
+grad_grad_kernel(int n_points, int n_levels, int n_all_levels, int levels_per_thread, uint32_t capacity, uint32_t cap_mask,
                  const float* __restrict__ positions, const T* __restrict__ table,
                  const float* __restrict__ scale_factor, const float* __restrict__ random_shift,
                  const float* __restrict__ window, const float* __restrict__ double_pos_grad,
                  float* __restrict__ grad_grad_sliced) {
     const int n = blockIdx.x * kBlock + threadIdx.x;
     if (n >= n_points) return;
-    const int level = blockIdx.y;
-    float* o = grad_grad_sliced + (static_cast<size_t>(level) * F) * n_points + n;
-    const float w_level = level < n_levels ? window[level] : 0.0f;  // concat levels: zeros (:1290-1295)
-    if (w_level == 0.0f) {
-        static_for<F>(PENC_BODY(k) {
-            PENC_INDEX(k); o[static_cast<size_t>(k) * n_points] = 0.0f; });
-        return;
-    }
-    const float* sf = scale_factor + level * D;
-    const Located<D> s = locate<D>(load_point<D>(positions, n), random_shift + level * D, sf);
-    // one trip through the thread's LDS column puts both the elevated gradient and the hash steps
-    // into rank order (as in the forward)
     __shared__ uint2 columns[(D + 1) * kBlock];
-    uvec<D + 1> h;
-    fvec<D + 1> sorted;
-    sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, pos_grad_grad_to_elevated<D>(load_point<D>(double_pos_grad, n), sf),
-                        s.hash0, sorted, h);
-    const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
-    // dB[r] * w_level, then times the vertex value (:1484-1485)
-    const fvec<D + 1> wr = sorted_elevated_grad_to_bary<D>(sorted) * w_level;
-    fvec<F> gg = 0.0f;
-    static_for<D + 1>(PENC_BODY(r) {
-        PENC_INDEX(r);
+    const fvec<D> point = load_point<D>(positions, n), q = load_point<D>(double_pos_grad, n);
+    // the levels of a thread are `gridDim.y` apart, as in the forward
+#pragma unroll 1
+    for (int k2 = 0; k2 < levels_per_thread; ++k2) {
+        const int level = static_cast<int>(blockIdx.y) + k2 * static_cast<int>(gridDim.y);
+        if (level >= n_all_levels) break;
+        float* o = grad_grad_sliced + (static_cast<size_t>(level) * F) * n_points + n;
+        const float w_level = level < n_levels ? window[level] : 0.0f;  // concat levels: zeros (:1290-1295)
+        if (w_level == 0.0f) {
+            static_for<F>(PENC_BODY(k) {
+                PENC_INDEX(k); o[static_cast<size_t>(k) * n_points] = 0.0f; });
+            continue;
+        }
+        const float* sf = scale_factor + level * D;
+        const Located<D> s = locate<D>(point, random_shift + level * D, sf);
+        // one trip through the thread's LDS column puts both the elevated gradient and the hash steps
+        // into rank order (as in the forward)
+        uvec<D + 1> h;
+        fvec<D + 1> sorted;
+        sort_by_rank_lds<D>(columns + threadIdx.x, kBlock, s.rank, pos_grad_grad_to_elevated<D>(q, sf), s.hash0, sorted, h);
+        const Vertices<D, F> v = load_vertices<D, F, T>(table + static_cast<size_t>(level) * capacity * F, h, capacity, cap_mask);
+        // dB[r] * w_level, then times the vertex value (:1484-1485)
+        const fvec<D + 1> wr = sorted_elevated_grad_to_bary<D>(sorted) * w_level;
+        fvec<F> gg = 0.0f;
+        static_for<D + 1>(PENC_BODY(r) {
+            PENC_INDEX(r);
+            static_for<F>(PENC_BODY(k) {
+                PENC_INDEX(k); gg[k] += wr[r] * v.f[k][r]; });
+        });
         static_for<F>(PENC_BODY(k) {
-            PENC_INDEX(k); gg[k] += wr[r] * v.f[k][r]; });
-    });
-    static_for<F>(PENC_BODY(k) {
-        PENC_INDEX(k); o[static_cast<size_t>(k) * n_points] = gg[k]; });
+            PENC_INDEX(k); o[static_cast<size_t>(k) * n_points] = gg[k]; });
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -753,6 +766,11 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
 
 inline unsigned tiles(int64_t n) { return static_cast<unsigned>((n + kBlock - 1) / kBlock); }
 
+// Levels a thread of the forward and of the gathering half of the double backward takes: two up to
+// pos_dim 4 (measured on the forward at 2^20 points, 24 levels: 0.310 -> 0.302 ms at pos_dim 3, 0.275 -> 0.259 ms with a
+// 2^22-slot table, 0.396 -> 0.392 ms at pos_dim 4; at pos_dim 8 0.283 -> 0.298 ms).
+inline int gather_levels_per_thread(int pos_dim) { return pos_dim <= 4 ? 2 : 1; }
+
 // Device address of this GPU's copy of `scratch`, looked up on the first call with that GPU
 // current and kept for the life of the process.  Returns nullptr when the lookup fails.
 constexpr int kMaxDevices = 64;
@@ -925,10 +943,11 @@ static int forward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_l
         return PENC_ERR_NULL_POINTER;
     if (!table_aligned(table, nr_feat)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 grid(tiles(nr_positions), nr_levels + extra);
+    const int per_thread = gather_levels_per_thread(pos_dim);
+    const dim3 grid(tiles(nr_positions), (nr_levels + extra + per_thread - 1) / per_thread);
     PENC_DISPATCH_DFT(pos_dim, nr_feat, table.format,
                       hipLaunchKernelGGL((forward_kernel<DD, FF, TT>), grid, dim3(kBlock), 0, st,
-                                         static_cast<int>(nr_positions), nr_levels, static_cast<uint32_t>(capacity),
+                                         static_cast<int>(nr_positions), nr_levels, nr_levels + extra, per_thread, static_cast<uint32_t>(capacity),
                                          mask_of(capacity), positions, static_cast<const TT*>(table.values), scale_factor,
                                          random_shift, anneal_window, sliced_values, points_scaling));
     return check_launch();
@@ -1154,10 +1173,11 @@ static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, 
     if (!table_aligned(table, nr_feat) || !aligned8(lattice_values_grad)) return PENC_ERR_MISALIGNED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (grad_grad_sliced_values) {
-        const dim3 grid(tiles(nr_positions), nr_levels + extra);
+        const int per_thread = gather_levels_per_thread(pos_dim);
+        const dim3 grid(tiles(nr_positions), (nr_levels + extra + per_thread - 1) / per_thread);
         PENC_DISPATCH_DFT(pos_dim, nr_feat, table.format,
                           hipLaunchKernelGGL((grad_grad_kernel<DD, FF, TT>), grid, dim3(kBlock), 0, st,
-                                             static_cast<int>(nr_positions), nr_levels, static_cast<uint32_t>(capacity),
+                                             static_cast<int>(nr_positions), nr_levels, nr_levels + extra, per_thread, static_cast<uint32_t>(capacity),
                                              mask_of(capacity), positions, static_cast<const TT*>(table.values), scale_factor,
                                              random_shift, anneal_window, double_positions_grad, grad_grad_sliced_values));
         if (int rc = check_launch()) return rc;
