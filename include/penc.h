@@ -123,8 +123,9 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
  *     (about 1.3 million points at pos_dim 3 and 2^18 slots, 0.7 million at 2^22 slots); larger problems return PENC_ERR_SCRATCH_TOO_SMALL
  *     and nothing is enqueued.  Levels are binned in as many passes as the scratch needs; position
  *     gradients whose partial sums do not fit are summed by one thread per point instead.
- *   - Every call on a GPU uses that GPU's one array, whose contents survive between calls; nothing
- *     in it has to start at zero (every count is written before it is read).  Calls that overlap on
+ *   - Every call on a GPU uses that GPU's one array, whose contents survive between calls; what
+ *     has to start at zero (a flag per level and slot range) is cleared by the call's own fill kernel,
+ *     and every count is written before it is read.  Calls that overlap on
  *     one GPU (two streams, two threads) race on it: serialise them. */
 #define PENC_STATIC_SCRATCH_BYTES (64u << 20)
 size_t penc_static_scratch_bytes(void);
