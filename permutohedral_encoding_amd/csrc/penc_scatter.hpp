@@ -57,7 +57,10 @@ constexpr int kCacheLines = 1 << kCacheLinesLog2;  // accumulate-cache lines per
 constexpr int kWaveGroups = 6;         // same-slot groups a wave folds with DPP before it touches the cache
 constexpr int kMinWaveGroup = 8;       // ... as long as the groups have at least this many lanes
 constexpr int kColumnMinIdsLog2 = 5;   // column mode: the cache's kCacheLines cells per feature are 32 columns of 64 cells (one per lane) ...
-constexpr int kColumnMaxIdsLog2 = 7;   // ... up to 128 columns of 16 cells, by the number of distinct slots the first tile has shown
+#ifndef PENC_COLUMN_MAX_IDS_LOG2
+#define PENC_COLUMN_MAX_IDS_LOG2 7
+#endif
+constexpr int kColumnMaxIdsLog2 = PENC_COLUMN_MAX_IDS_LOG2;   // ... up to 128 columns of 16 cells, by the number of distinct slots the first tile has shown
 constexpr int kColumnProbes = 16;      // linear probes before a contribution gives up on the column table
 enum ScatterMode : int { kModeCache = 0, kModeStream = 1, kModeColumns = 2 };
 // vertices per thread a wave sorts by bin in one go (256 or 320 records): all D+1 of them up to D = 4
@@ -325,13 +328,15 @@ __device__ __forceinline__ bool append_record(State& c, const BinTarget& bins, u
 // line already held the slot (a hit, as opposed to a claim).
 // (Spreading the lanes that share a slot over replicated sub-tables, instead of folding them in
 // registers first, was measured 30% slower on the coarse levels, and no faster on top of folding.)
-template <typename State>
+template <int kProbes = 2, typename State>
 __device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) {
     const int want = static_cast<int>(slot);
     int e = static_cast<int>(slot & (kCacheLines - 1));
     found = false;
+    constexpr uint32_t kMix[3] = {0x9E3779B1u, 0x85EBCA6Bu, 0xC2B2AE35u};
+    static_assert(kProbes >= 1 && kProbes <= 4, "one mixing constant per probe after the first");
 #pragma unroll
-    for (int probe = 0; probe < 2; ++probe) {
+    for (int probe = 0; probe < kProbes; ++probe) {
         int owner = c.tag[e];
         if (owner == want) {
             found = true;
@@ -341,7 +346,7 @@ __device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) 
             owner = atomicCAS(&c.tag[e], -1, want);
             if (owner == -1 || owner == want) return e;
         }
-        e = static_cast<int>((slot * 0x9E3779B1u) >> (32 - kCacheLinesLog2));
+        if (probe + 1 < kProbes) e = static_cast<int>((slot * kMix[probe]) >> (32 - kCacheLinesLog2));
     }
     return -1;
 }
@@ -799,7 +804,16 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
             }
             bool found = false;
             if (miss) {
-                const int e = cache_find(c, slot[r], found);
+                // From D = 4 on a third candidate line: every contribution of a slot that finds no line becomes
+                // a record, and tens of thousands of records on a handful of slots serialise in the LDS of
+                // the one reducer workgroup that owns their bin.  At D = 3 the low 11 bits of a coarse level's
+                // slots are all distinct and two candidates leave no slot out while the level fits; at D = 4
+                // they collide (levels 6 and 7 of 24: 350 and 1000 slots, 4 and 110 of them left out; those
+                // levels' reducer workgroups took 0.05-0.11 ms each, and with a third candidate the
+                // double backward's table half went from 0.73 to 0.65 ms; at D = 3 it would add 2% to the
+                // scattering kernel for nothing).
+                constexpr int kProbes = D >= 4 ? 3 : 2;
+                const int e = cache_find<kProbes>(c, slot[r], found);
                 if (e >= 0) {
                     __hip_atomic_fetch_add(&c.val[0][e], static_cast<double>(x0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                     __hip_atomic_fetch_add(&c.val[1][e], static_cast<double>(x1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
