@@ -168,6 +168,17 @@ forward_kernel(int n_points, int n_levels, int n_all_levels, int levels_per_thre
 // ------------------------------------------------------------------------------------------
 // backward w.r.t. the table (EncodingGPU.cuh:259-414)
 
+// Wavefronts per SIMD the scattering kernel is compiled for: six (three workgroups per compute unit, at
+// most 80 vector registers) where that costs a few spilled registers at most, else four (two
+// workgroups, 128 registers).  Measured at 2^19 points, 24 levels: table backward 0.367 -> 0.338 ms
+// at D = 4 (84 -> 80 registers, 3 spilled), 0.458 -> 0.424 ms at D = 5; the second-order kernel
+// 0.577 -> 0.552 ms at D = 4, but 0.735 -> 0.754 ms at D = 5 (11 spilled), which therefore stays at
+// four; at D = 8 the second-order kernel needed 130 registers and ran one workgroup per compute
+// unit: held to 128, 1.334 -> 1.113 ms.
+constexpr int scatter_waves_per_simd(int pos_dim, bool second_order) {
+    return pos_dim <= 4 || (pos_dim == 5 && !second_order) ? 6 : 4;
+}
+
 // kRowMajor: the upstream gradient is read as rows grad[n][2*level + feature] of `grad_row_stride`
 // floats (what the layer after the encoding produces) instead of [level][feature][n].  A die walks
 // all levels of a group of points back to back, so the rows mostly come from L2 (measured: fetched
@@ -183,7 +194,7 @@ forward_kernel(int n_points, int n_levels, int n_all_levels, int levels_per_thre
 // `pair_level` = level * feat_pairs + pair.  The upstream gradient needs no special case: [L][F][N]
 // is [L * F/2][2][N], and in a row the pair sits at column 2 * pair_level.
 template <int D, bool kRowMajor, bool kSecondOrder>
-__global__ void __launch_bounds__(kScatterBlock)
+__global__ void __launch_bounds__(kScatterBlock, scatter_waves_per_simd(D, kSecondOrder))
 backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t feat_pairs, uint32_t dies, int tiles_per_group,
                       uint32_t capacity, uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
