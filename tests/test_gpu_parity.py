@@ -749,16 +749,23 @@ def test_many_bins_levels_shared_by_a_reducer_workgroup(feat, cap, levels, n):
     between, coarse levels whose scattering workgroups add straight into the gradient (so the
     reducer must add to what is there), and one slot range past a power of two.  First- and
     second-order table gradients against the oracle."""
+    from permutohedral_encoding_amd import _native
     d = 3
     p = random_problem(d, n, levels, cap, seed=300 + levels, sigma_range=(1.0, 2e-3), nr_feat=feat)
     p["window"][[1, levels - 2]] = 0.0
     sf = orc.scale_factors(d, p["sigmas"])
     enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
     inp = gpu_input(p, need_pos_grad=False)
-    tg, _ = enc.backward(inp, to_gpu(p["grad"]))
     want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
-    assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "table gradient")
-    assert not tg[1].any() and not tg[levels - 2].any()
+    full = _native.lib().penc_scatter_workspace_bytes(d, n, levels * feat // 2, cap, 0)
+    for limit in (None, full // 3):  # all levels in one pass; several passes, each with its own share of the flags
+        _native.MAX_WORKSPACE_BYTES = limit
+        try:
+            tg, _ = enc.backward(inp, to_gpu(p["grad"]))
+        finally:
+            _native.MAX_WORKSPACE_BYTES = None
+        assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, workspace cap {limit}")
+        assert not tg[1].any() and not tg[levels - 2].any()
     tg2, _ = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
     want = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
     assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "second-order table gradient")
