@@ -19,7 +19,7 @@
 //      add without meeting each other, and the wave-wide folding that a handful of hot lines
 //      needs, which is what bounds those levels (vector ALU), is not needed at all.
 //   2. Slot-range bins (optional, needs a workspace).  A contribution that finds no line in the
-//      cache is appended, as a 12-byte record, to the bin of its slot range (each workgroup has a
+//      cache is appended, as a record of 12 or 10 bytes, to the bin of its slot range (each workgroup has a
 //      private segment in every bin, so appending costs one LDS counter increment and one
 //      store); a second kernel (bin_reduce_kernel) reads each bin back coalesced, sums it in
 //      LDS (fp64), and adds the range into the gradient with coalesced read-modify-writes.  This
@@ -27,7 +27,7 @@
 //      look-up of the first tile's slots shows that the cache would not hit at its level never
 //      fills it: the cache's LDS becomes staging space in which the records of a tile are sorted by
 //      bin, so that records of one bin leave in runs of consecutive addresses (whole cache lines)
-//      instead of one 12-byte store each.
+//      instead of one small store each.
 //   3. Direct global atomics, with the two features of a slot in one instruction (lane pairs),
 //      for whatever is left: no workspace, capacity too large for binning, or a full bin.
 // The result never depends on a stage hitting: every stage falls through to the next.
@@ -571,7 +571,7 @@ __device__ __forceinline__ void stream_tile_many(State& c, const GradSlice& leve
 // counts its records per bin (one LDS counter per bin, owned by one lane), reserves room for each
 // bin's run in the workgroup's segment with one add per bin, lays the records out bin by bin in
 // its slice, and then stores them in that order: neighbouring lanes write neighbouring addresses.
-// A staged record carries its destination (byte offset / 12 in the level's record array), so the
+// A staged record carries its destination (its index in the level's record array), so the
 // store needs no search.  When a run does not fit its segment any more (rare: the segments hold
 // the mean plus three standard deviations) the whole chunk takes the careful path, which checks
 // every record against the room left and sends the excess to stage 3.
