@@ -720,7 +720,7 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
         p.target.segment_capacity <= kLevelsMaxSegment && p.target.n_groups <= static_cast<uint32_t>(kReduceBlock)) {
         const unsigned levels = static_cast<unsigned>(n_levels_in_pass);
         unsigned per_bin = (levels + kLevelsMaxPerWorkgroup - 1) / kLevelsMaxPerWorkgroup;
-        const unsigned to_fill = (2 * kReduceWorkgroupsWanted + p.target.n_bins - 1) / p.target.n_bins;  // four workgroups per compute unit, one after the other
+        const unsigned to_fill = (kReduceWorkgroupsWanted + p.target.n_bins - 1) / p.target.n_bins;  // two workgroups per compute unit, one after the other
         if (per_bin < to_fill) per_bin = to_fill;
         if (per_bin > levels) per_bin = levels;
         hipLaunchKernelGGL(bin_reduce_levels_kernel, dim3(p.target.n_bins, per_bin), dim3(kReduceBlock), 0, st, p.target, window,

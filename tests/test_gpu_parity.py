@@ -745,7 +745,7 @@ def test_segments_overflow_with_more_bins_than_lanes():
 def test_many_bins_levels_shared_by_a_reducer_workgroup(feat, cap, levels, n):
     """Tables with hundreds of slot ranges, whose segments hold a few dozen records, are reduced by
     workgroups that keep their range and walk several levels: level lists that divide unevenly among
-    them (26 pairs of features over 4 workgroups, 7 levels over 4, 16 over 2), masked levels in
+    them (26 pairs of features over 2 workgroups, 7 levels over 2, 16 in one), masked levels in
     between, coarse levels whose scattering workgroups add straight into the gradient (so the
     reducer must add to what is there), and one slot range past a power of two.  First- and
     second-order table gradients against the oracle."""
