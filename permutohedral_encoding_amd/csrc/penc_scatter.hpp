@@ -1029,9 +1029,13 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
         struct Cursor {
             uint32_t k, base;  // segment (of this wave's n_segments), first record of the chunk
         };
+        // (Past the last chunk the loads are issued all the same, from the wave's first segment: with loads
+        // behind a branch the compiler cannot tell how many are on their way when the other chunk is added, and
+        // makes the adds wait for all of them.)
         const auto fetch = [&](const Cursor& at, Loaded& got) {
-            const uint32_t count = count_of(at.k);
-            const size_t seg = first + (g0 + at.k * kWaves) * bins.segment_capacity;
+            const bool any = at.k < n_segments;
+            const uint32_t count = any ? count_of(at.k) : 0u;
+            const size_t seg = first + (g0 + (any ? at.k : 0u) * kWaves) * bins.segment_capacity;
             if constexpr (kSplit) {
                 const RecordValues* values = static_cast<const RecordValues*>(bins.records) + seg;  // 16-byte aligned:
                 const uint16_t* slots = bins.slots + seg;                                         // segments are multiples of four records
@@ -1092,11 +1096,11 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
         if (a.k < n_segments) fetch(a, got_a);
         while (a.k < n_segments) {
             const Cursor b = after(a);
-            if (b.k < n_segments) fetch(b, got_b);
+            fetch(b, got_b);
             add(a, got_a);
             if (b.k >= n_segments) break;
             a = after(b);
-            if (a.k < n_segments) fetch(a, got_a);
+            fetch(a, got_a);
             add(b, got_b);
         }
     }
