@@ -72,9 +72,10 @@ int penc_scale_factors(int pos_dim, int nr_levels, const float* sigmas, float* s
 
 /* Suggested size of the `workspace` argument of the gradient calls below for binning
  * `levels_per_pass` levels at a time (<= 0: the library's default, all of them); 0 when the capacity
- * is too large for binning (above 2^22 slots).  `nr_levels` counts pairs of features: pass
+ * is too large for binning (above 2^25 slots).  `nr_levels` counts pairs of features: pass
  * nr_levels * nr_feat / 2.  Per level the workspace holds, for each of the ceil(capacity / 8192)
- * slot ranges and each group of 4096 or 8192 points, a 4-byte count and room for the group's
+ * slot ranges (at most 512: above 2^22 slots a range spans 2^14 to 2^16 slots) and each group of
+ * 4096 or 8192 points, a 4-byte count and room for the group's
  * expected share of the (pos_dim + 1) records per point plus three standard deviations; a record is
  * 10 bytes for pos_dim <= 5 and capacities up to 2^19 and 12 bytes otherwise: about 11.5 or
  * 13.5 * (pos_dim + 1) bytes per point and level (1.2 GiB for 2^20 points, 24 levels, pos_dim 3).

@@ -175,7 +175,8 @@ forward_kernel(int n_points, int n_levels, int n_all_levels, int levels_per_thre
 // 0.577 -> 0.552 ms at D = 4, but 0.735 -> 0.754 ms at D = 5 (11 spilled), which therefore stays at
 // four; at D = 8 the second-order kernel needed 130 registers and ran one workgroup per compute
 // unit: held to 128, 1.334 -> 1.113 ms.
-constexpr int scatter_waves_per_simd(int pos_dim, bool second_order) {
+constexpr int scatter_waves_per_simd(int pos_dim, bool second_order, bool wide_bins) {
+    if (wide_bins) return pos_dim <= 3 ? 6 : 4;  // (a variable bin width takes six to eight more registers: up to 30 spilled at D = 4)
     return pos_dim <= 4 || (pos_dim == 5 && !second_order) ? 6 : 4;
 }
 
@@ -193,8 +194,11 @@ constexpr int scatter_waves_per_simd(int pos_dim, bool second_order) {
 // share their geometry: "levels" below (first_level, n_pass_levels, the grid, the bins) count pairs,
 // `pair_level` = level * feat_pairs + pair.  The upstream gradient needs no special case: [L][F][N]
 // is [L * F/2][2][N], and in a row the pair sits at column 2 * pair_level.
-template <int D, bool kRowMajor, bool kSecondOrder>
-__global__ void __launch_bounds__(kScatterBlock, scatter_waves_per_simd(D, kSecondOrder))
+// kWideBins: the bins span more than kBinSlots slots (tables above 2^22 slots).  A parameter of the kernel
+// rather than a value read from its arguments, because with the bin width a variable the usual instances
+// need up to eight more vector registers (at D = 4, held to 80 registers, 27 spilled instead of 5).
+template <int D, bool kRowMajor, bool kSecondOrder, bool kWideBins>
+__global__ void __launch_bounds__(kScatterBlock, scatter_waves_per_simd(D, kSecondOrder, kWideBins))
 backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uint32_t feat_pairs, uint32_t dies, int tiles_per_group,
                       uint32_t capacity, uint32_t cap_mask,
                       const float* __restrict__ positions, const float* __restrict__ scale_factor,
@@ -218,9 +222,10 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     const float w_level = window[level];
     if (w_level == 0.0f) return;
     scatter_begin(state);
-    const BinTarget bins = bins_of_level(pass_bins, level_in_pass);
+    BinTarget bins = bins_of_level(pass_bins, level_in_pass);
+    if constexpr (!kWideBins) bins.bin_shift = kBinSlotsLog2;  // a constant from here on
     const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair_level % feat_pairs) * 2,
-                               2 * feat_pairs, bins.records != nullptr ? bins.direct : nullptr};
+                               2 * feat_pairs, bins.records != nullptr ? bins.direct : nullptr, bins.bin_shift};
     // Everything a thread reads lies within its group of at most 16 x 512 points, so the addresses are
     // wave-uniform 64-bit bases (scalar registers) plus 32-bit per-thread offsets.
     const uint32_t last_in_group = static_cast<uint32_t>(n_points - 1 - group_base);
@@ -615,8 +620,20 @@ inline size_t direct_flag_bytes(int levels, uint32_t n_bins) {
     return (static_cast<size_t>(levels) * n_bins * sizeof(uint32_t) + 255u) & ~size_t{255};
 }
 
+// log2 of the slots per bin: kBinSlotsLog2 (what a reducer workgroup's LDS holds) up to kMaxBins bins, wider
+// bins (summed one LDS-full after the other) for larger tables, up to kMaxBinSlotsLog2.
+inline uint32_t bin_shift_for_capacity(int capacity) {
+    uint32_t shift = kBinSlotsLog2;
+    while (shift < static_cast<uint32_t>(kMaxBinSlotsLog2) &&
+           ((static_cast<int64_t>(capacity) + (int64_t{1} << shift) - 1) >> shift) > kMaxBins)
+        ++shift;
+    return shift;
+}
+
+// Bins per level; more than kMaxBins means the table is too large for binning.
 inline uint32_t bins_for_capacity(int capacity) {
-    return static_cast<uint32_t>((static_cast<int64_t>(capacity) + kBinSlots - 1) >> kBinSlotsLog2);
+    const uint32_t shift = bin_shift_for_capacity(capacity);
+    return static_cast<uint32_t>((static_cast<int64_t>(capacity) + (int64_t{1} << shift) - 1) >> shift);
 }
 
 constexpr int64_t kMinSlotsPerContribution = 8;
@@ -688,9 +705,14 @@ inline BinPlan plan_bins(int pos_dim, int64_t n, int levels, int capacity, int t
     }
     const size_t fit = bytes / bin_bytes_per_level(pos_dim, n_bins, n_groups, cap);
     p.levels_per_pass = static_cast<int>(fit < static_cast<size_t>(levels) ? fit : static_cast<size_t>(levels));
+    // wide bins are served by bin_reduce_levels_kernel only
+    if (bin_shift_for_capacity(capacity) != static_cast<uint32_t>(kBinSlotsLog2) &&
+        (cap > kLevelsMaxSegment || n_groups > static_cast<uint32_t>(kReduceBlock)))
+        return p;
     p.target.n_bins = n_bins;
     p.target.n_groups = n_groups;
     p.target.segment_capacity = cap;
+    p.target.bin_shift = bin_shift_for_capacity(capacity);
     p.target.direct = reinterpret_cast<uint32_t*>(base);
     p.direct_bytes = flag_bytes;
     const uintptr_t counts_at = base + flag_bytes;
@@ -716,8 +738,10 @@ inline int reduce_bins(const BinPlan& p, const float* window, int first_level, i
     if (splits > p.target.n_groups) splits = p.target.n_groups;
     if (splits > kMaxReduceSplits) splits = kMaxReduceSplits;
     // many bins with a few thousand records each: workgroups that keep their bin and walk several levels
-    if (p.target.slots == nullptr && p.target.n_bins > static_cast<uint32_t>(kStageBins) && splits == 1 &&
-        p.target.segment_capacity <= kLevelsMaxSegment && p.target.n_groups <= static_cast<uint32_t>(kReduceBlock)) {
+    // (bins wider than kBinSlots are planned only where this kernel can serve them)
+    const bool wide = p.target.bin_shift != static_cast<uint32_t>(kBinSlotsLog2);
+    if (wide || (p.target.slots == nullptr && p.target.n_bins > static_cast<uint32_t>(kStageBins) && splits == 1 &&
+                 p.target.segment_capacity <= kLevelsMaxSegment && p.target.n_groups <= static_cast<uint32_t>(kReduceBlock))) {
         const unsigned levels = static_cast<unsigned>(n_levels_in_pass);
         unsigned per_bin = (levels + kLevelsMaxPerWorkgroup - 1) / kLevelsMaxPerWorkgroup;
         const unsigned to_fill = (kReduceWorkgroupsWanted + p.target.n_bins - 1) / p.target.n_bins;  // two workgroups per compute unit, one after the other
@@ -840,8 +864,12 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
     // every pair of features is scattered like a level of its own (see backward_table_kernel)
     const uint32_t feat_pairs = static_cast<uint32_t>(nr_feat / 2);
     const int pair_levels = nr_levels * static_cast<int>(feat_pairs);
-    const int tiles_per_group = table_backward_tiles(nr_positions, pair_levels);
+    int tiles_per_group = table_backward_tiles(nr_positions, pair_levels);
     BinPlan plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
+    if (!plan.enabled && tiles_per_group != kScatterTiles) {  // wide bins need short segments: smaller groups of points
+        tiles_per_group = kScatterTiles;
+        plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
+    }
     if (int rc = clear_table_grad(lattice_values_grad, pair_levels, capacity, plan.enabled ? plan.target.direct : nullptr,
                                   plan.direct_bytes, st))
         return rc;
@@ -853,12 +881,19 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
         const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + dies - 1) / dies * dies;
         const dim3 grid(padded_groups * static_cast<unsigned>(count));
         if (plan.enabled) plan.target.direct = direct_flags + static_cast<size_t>(first) * plan.target.n_bins;
-#define PENC_LAUNCH_TABLE(ROW_MAJOR, SECOND_ORDER)                                                                         \
-    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER>), grid,                  \
+#define PENC_LAUNCH_TABLE_(ROW_MAJOR, SECOND_ORDER, WIDE)                                                                  \
+    PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER, WIDE>), grid,            \
                                                 dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
                                                 feat_pairs, dies, tiles_per_group, cap, mask, positions, scale_factor,       \
                                                 random_shift, anneal_window, grad, grad_row_stride, double_pos_grad,         \
                                                 lattice_values_grad, grad_level_major, plan.target))
+#define PENC_LAUNCH_TABLE(ROW_MAJOR, SECOND_ORDER)       \
+    if (wide_bins) {                                     \
+        PENC_LAUNCH_TABLE_(ROW_MAJOR, SECOND_ORDER, true);  \
+    } else {                                             \
+        PENC_LAUNCH_TABLE_(ROW_MAJOR, SECOND_ORDER, false); \
+    }
+        const bool wide_bins = plan.enabled && plan.target.bin_shift != static_cast<uint32_t>(kBinSlotsLog2);
         if (double_pos_grad != nullptr && grad_row_stride != 0) {
             PENC_LAUNCH_TABLE(true, true);
         } else if (double_pos_grad != nullptr) {
@@ -869,6 +904,7 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
             PENC_LAUNCH_TABLE(false, false);
         }
 #undef PENC_LAUNCH_TABLE
+#undef PENC_LAUNCH_TABLE_
         if (int rc = check_launch()) return rc;
         if (plan.enabled)
             if (int rc = reduce_bins(plan, anneal_window, first, count, capacity, feat_pairs, lattice_values_grad, st)) return rc;

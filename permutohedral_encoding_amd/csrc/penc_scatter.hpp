@@ -69,7 +69,9 @@ constexpr int kStageBins = 64;         // a wave counts one bin per lane: stagin
 constexpr int kWorkgroupSortMaxDim = 5;  // up to this input dimension a streaming workgroup sorts a tile's records across all its waves
 constexpr int kBinSlotsLog2 = 13;      // slots per bin: 8192 (128 KiB of fp64 sums in LDS)
 constexpr int kBinSlots = 1 << kBinSlotsLog2;
-constexpr int kMaxBins = 512;          // bins per level; capacities above kMaxBins*kBinSlots (2^22) are not binned
+constexpr int kMaxBins = 512;          // bins per level
+constexpr int kMaxBinSlotsLog2 = 16;   // tables of more than kMaxBins * kBinSlots slots (2^22) get bins of up to 2^16 slots, which their
+                                       // reducer sums one range of kBinSlots slots after the other; above 2^25 slots nothing is binned
 constexpr int kReduceBlock = 1024;     // threads of a bin_reduce_kernel workgroup
 
 // A contribution on its way through a bin: the slot within the bin's range and the two values.
@@ -107,6 +109,7 @@ struct BinTarget {
     uint32_t n_bins;
     uint32_t n_groups;
     uint32_t segment_capacity;
+    uint32_t bin_shift;  // log2 of the slots per bin: kBinSlotsLog2, more only with more than kStageBins bins (whole records)
 };
 
 // `pass` describes the first level of a launch; level k of the launch follows k bin arrays later.
@@ -190,9 +193,10 @@ struct GradSlice {
     float* base;
     uint32_t slot_floats;
     uint32_t* direct;
+    uint32_t bin_shift;  // of the bins `direct` belongs to
     __device__ __forceinline__ float* at(uint32_t slot) const { return base + static_cast<size_t>(slot) * slot_floats; }
     __device__ __forceinline__ void mark_direct(uint32_t slot) const {
-        if (direct != nullptr) direct[slot >> kBinSlotsLog2] = 1u;
+        if (direct != nullptr) direct[slot >> bin_shift] = 1u;
     }
 };
 
@@ -314,10 +318,10 @@ __device__ __forceinline__ void scatter_begin(State& c) {
 template <typename State>
 __device__ __forceinline__ bool append_record(State& c, const BinTarget& bins, uint32_t group, uint32_t slot,
                                               float a0, float a1) {
-    const uint32_t b = slot >> kBinSlotsLog2;
+    const uint32_t b = slot >> bins.bin_shift;
     const uint32_t pos = atomicAdd(&c.bin_count[b], 1u);
     if (pos >= bins.segment_capacity) return false;
-    store_record(bins, (b * bins.n_groups + group) * bins.segment_capacity + pos, slot & (kBinSlots - 1), a0, a1);
+    store_record(bins, (b * bins.n_groups + group) * bins.segment_capacity + pos, slot & ((1u << bins.bin_shift) - 1u), a0, a1);
     return true;
 }
 
@@ -497,7 +501,7 @@ __device__ __forceinline__ void stream_tile_many(State& c, const GradSlice& leve
         uvec<kStageChunk> place = 0u;  // rank of each record within the workgroup's run for its bin
         static_for<kCount>(PENC_BODY(j) {
             PENC_INDEX(j);
-            if (active) place[j] = atomicAdd(&count[slot[kFirst + j] >> kBinSlotsLog2], 1u);
+            if (active) place[j] = atomicAdd(&count[slot[kFirst + j] >> bins.bin_shift], 1u);
         });
         __syncthreads();
         uint32_t mine = 0u;
@@ -528,7 +532,7 @@ __device__ __forceinline__ void stream_tile_many(State& c, const GradSlice& leve
         static_for<kCount>(PENC_BODY(j) {
             PENC_INDEX(j);
             if (active) {
-                const uint32_t b = slot[kFirst + j] >> kBinSlotsLog2;
+                const uint32_t b = slot[kFirst + j] >> bins.bin_shift;
                 // copies first: a bit cast applied directly to a vector element reads element 0
                 const float v0 = a0[kFirst + j], v1 = a1[kFirst + j];
                 const uint32_t to = dest[b] + place[j];
@@ -550,7 +554,7 @@ __device__ __forceinline__ void stream_tile_many(State& c, const GradSlice& leve
             if (i < total) {
                 e = stage[i];
                 if (e.w != kNoRoom) {
-                    store_record(bins, e.w, e.x & (kBinSlots - 1), __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
+                    store_record(bins, e.w, e.x & ((1u << bins.bin_shift) - 1u), __builtin_bit_cast(float, e.y), __builtin_bit_cast(float, e.z));
                 } else {
                     spill = true;  // the segment is full: stage 3
                 }
@@ -1105,8 +1109,8 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
         }
     }
     __syncthreads();
-    const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr};
-    const uint32_t slot0 = bin << kBinSlotsLog2;
+    const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr, 0u};
+    const uint32_t slot0 = bin << kBinSlotsLog2;  // (this kernel serves bins of kBinSlots slots only)
     const bool alone = gridDim.z == 1;
     if (alone) {
         // nothing but this workgroup has added to the bin's slots since the gradient was cleared: the sums are the result
@@ -1219,14 +1223,19 @@ bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, 
 
     // a step: 64 segments of one level, one per quarter wave
     constexpr uint32_t kEnd = 32;
+    // Bins wider than the LDS sums (tables above 2^22 slots) are summed one range of kBinSlots slots after
+    // the other: every range walks all the bin's records and takes those that fall into it.
+    const uint32_t n_ranges = 1u << (pass_bins.bin_shift - kBinSlotsLog2);
     struct Cursor {
-        uint32_t i, step;  // the workgroup's i-th level (kEnd: past the last), segments 64 * step ...
+        uint32_t i, range, step;  // the workgroup's i-th level (kEnd: past the last), the range of the bin, segments 64 * step ...
     };
     const uint32_t n_steps = (n_groups + 63) / 64;
     const auto after = [&](Cursor at) {
         if (++at.step < n_steps) return at;
+        at.step = 0u;
+        if (++at.range < n_ranges) return at;
         const uint32_t rest = at.i + 1 < 32 ? todo >> (at.i + 1) : 0u;
-        return Cursor{rest != 0u ? at.i + 1 + static_cast<uint32_t>(__builtin_ctz(rest)) : kEnd, 0u};
+        return Cursor{rest != 0u ? at.i + 1 + static_cast<uint32_t>(__builtin_ctz(rest)) : kEnd, 0u, 0u};
     };
     const uint32_t reader = wave * 4 + lane / kLevelsShortLanes, l = lane % kLevelsShortLanes;
     // (Every load below is issued whether or not its result is wanted, from an address that is valid
@@ -1240,13 +1249,14 @@ bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, 
     };
     struct Loaded {
         RecordWords rec[kLevelsShortUnroll];
-        uint32_t count;
+        uint32_t count, range;
     };
     const BinRecord* const records = static_cast<const BinRecord*>(pass_bins.records);
     const auto fetch = [&](const Cursor& at, uint32_t count, Loaded& got) {
         const uint32_t g = at.step * 64 + reader;
         const BinRecord* seg = records + (first_segment(at.i != kEnd ? at.i : 0u) + (g < n_groups ? g : 0u)) * seg_cap;
         got.count = count;
+        got.range = at.range;
 #pragma unroll
         for (uint32_t u = 0; u < kLevelsShortUnroll; ++u) {
             const uint32_t idx = u * kLevelsShortLanes + l;
@@ -1259,21 +1269,22 @@ bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, 
         for (uint32_t u = 0; u < kLevelsShortUnroll; ++u) {
             const RecordWords w = got.rec[u];
             const uint32_t w0 = w.x, w1 = w.y, w2 = w.z;  // copies first: a bit cast applied directly to a vector element reads element 0
-            if (u * kLevelsShortLanes + l < got.count) {
-                __hip_atomic_fetch_add(&acc0[w0], static_cast<double>(__builtin_bit_cast(float, w1)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                __hip_atomic_fetch_add(&acc1[w0], static_cast<double>(__builtin_bit_cast(float, w2)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (u * kLevelsShortLanes + l < got.count && (w0 >> kBinSlotsLog2) == got.range) {
+                const uint32_t cell = w0 & (kBinSlots - 1);
+                __hip_atomic_fetch_add(&acc0[cell], static_cast<double>(__builtin_bit_cast(float, w1)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                __hip_atomic_fetch_add(&acc1[cell], static_cast<double>(__builtin_bit_cast(float, w2)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
         }
     };
-    // Adds the sums of the workgroup's i-th level into the gradient and clears them.  Nothing else touches
+    // Adds the sums of one range of the bin at the workgroup's i-th level into the gradient and clears them.  Nothing else touches
     // the bin's slots of that level while this kernel runs, so the add is a plain read-modify-write, or a
     // store where nothing was added since the gradient was cleared.
-    const auto flush = [&](uint32_t i) {
+    const auto flush = [&](uint32_t i, uint32_t range) {
         lds_barrier();
         const uint32_t pair_level = static_cast<uint32_t>(first_level) + level_in_pass(i);
         const uint32_t level = pair_level / feat_pairs, pair = pair_level % feat_pairs;
-        const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr};
-        const uint32_t slot0 = bin << kBinSlotsLog2;
+        const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr, 0u};
+        const uint32_t slot0 = (bin << pass_bins.bin_shift) + (range << kBinSlotsLog2);
         const bool untouched_so_far = ((direct_mask >> i) & 1u) == 0u;
         constexpr int kMine = kBinSlots / kReduceBlock;
         // (two loops, so that the usual one has no load to wait for: a wait would also be one for the
@@ -1312,7 +1323,7 @@ bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, 
     };
     // two sets of registers take turns for the records, two registers for the counts; past the last step the
     // counts are zero and the loads fetch the stand-in
-    Cursor it0{static_cast<uint32_t>(__builtin_ctz(todo)), 0u};
+    Cursor it0{static_cast<uint32_t>(__builtin_ctz(todo)), 0u, 0u};
     Cursor it1 = after(it0);
     uint32_t count_x = load_count(it0), count_y = load_count(it1);
     Loaded got_a, got_b;
@@ -1322,13 +1333,13 @@ bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, 
         count_x = load_count(it2);
         fetch(it1, count_y, got_b);
         add(got_a);
-        if (it1.i != it0.i) flush(it0.i);
+        if (it1.i != it0.i || it1.range != it0.range) flush(it0.i, it0.range);
         if (it1.i == kEnd) break;
         const Cursor it3 = it2.i != kEnd ? after(it2) : it2;
         count_y = load_count(it3);
         fetch(it2, count_x, got_a);
         add(got_b);
-        if (it2.i != it1.i) flush(it1.i);
+        if (it2.i != it1.i || it2.range != it1.range) flush(it1.i, it1.range);
         if (it2.i == kEnd) break;
         it0 = it2;
         it1 = it3;

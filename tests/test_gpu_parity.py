@@ -771,6 +771,34 @@ def test_many_bins_levels_shared_by_a_reducer_workgroup(feat, cap, levels, n):
     assert_sum_close(tg2.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "second-order table gradient")
 
 
+@pytest.mark.parametrize("cap,n,feat", [(1 << 23, 300000, 2), (5_000_011, 200000, 2), (1 << 25, 1 << 20, 2), (1 << 23, 300000, 4)])
+def test_tables_above_2_22_slots_get_wider_bins(cap, n, feat):
+    """Above 2^22 slots a bin spans 2^14 to 2^16 slots and its reducer workgroup sums it one range of 2^13
+    slots after the other (up to 2^25 slots: 512 bins of 2^16).  Coarse levels that add straight
+    into the gradient, a masked level, a capacity that is no power of two, four features; first- and
+    second-order table gradients against the oracle.  (The oracle's sums are compared level by level:
+    at 2^25 slots one level's fp64 sums are 1 GiB.)"""
+    from permutohedral_encoding_amd import _native
+    d, levels = 3, 5
+    assert _native.lib().penc_scatter_workspace_bytes(d, n, levels * feat // 2, cap, 0) > 0
+    p = random_problem(d, n, levels, 1, seed=41 + feat, sigma_range=(0.3, 2e-3), nr_feat=feat)
+    p["window"][1] = 0.0
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
+    table = torch.zeros(levels, cap, feat, device="cuda")  # the table gradient does not read the table
+    inp = _native.EncodingInput(table, to_gpu(p["pos"]), to_gpu(p["window"]), True, False)
+    tg, _ = enc.backward(inp, to_gpu(p["grad"]))
+    tg2, _ = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    assert not tg[1].any() and not tg2[1].any()
+    for level in range(levels):
+        one = slice(level, level + 1)
+        args = (p["pos"], sf[one], p["shift"][one], p["window"][one])
+        want = orc.backward_table(*args, p["grad"][one], cap, want_abs=True)
+        assert_sum_close(tg[level].cpu().numpy()[None], want["grad64"], want["abs64"], SUM_RTOL, f"table gradient, level {level}")
+        want = orc.double_backward(p["pos"], np.zeros((1, cap, feat), np.float32), sf[one], p["shift"][one], p["window"][one], p["dpos"], p["grad"][one], want_abs=True)
+        assert_sum_close(tg2[level].cpu().numpy()[None], want["grad64"], want["abs64"], SUM_RTOL, f"second-order table gradient, level {level}")
+
+
 def test_records_crowd_one_bin():
     """Points chosen so that, at the finest level, at least three of their four vertices fall into the
     first of four slot ranges: the tile's records are all distinct (the workgroup streams them sorted
