@@ -92,7 +92,9 @@ def test_argument_validation_without_a_gpu():
     w4 = lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 4)
     assert 0 < w1 < w4 <= 4 * w1 and lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 100) <= 24 * w1
     assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 22, 4) > 0
-    assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, (1 << 22) + 1, 4) == 0
+    assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, (1 << 22) + 1, 4) > 0  # wider slot ranges up to 2^25 slots
+    assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 25, 4) > 0
+    assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, (1 << 25) + 1, 4) == 0
     assert lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 0) == lib.penc_scatter_workspace_bytes(3, 1 << 20, 24, 1 << 18, 24)
 
 
