@@ -799,6 +799,16 @@ def test_tables_above_2_22_slots_get_wider_bins(cap, n, feat):
         assert_sum_close(tg2[level].cpu().numpy()[None], want["grad64"], want["abs64"], SUM_RTOL, f"second-order table gradient, level {level}")
 
 
+@pytest.mark.parametrize("n", [(1 << 15) + 5, (1 << 16) + 77, (1 << 17) + 1])
+def test_small_batches_take_smaller_groups(n):
+    """Below 2^17 points (24 levels) the scattering workgroups take groups of two or four tiles instead of
+    eight, so that the launch still fills the chip; the headline geometry at those sizes, first- and
+    second-order table gradients against the oracle."""
+    d, levels, cap = 3, 24, 1 << 18
+    p = random_problem(d, n, levels, cap, seed=n % 1000, sigma_range=(1.0, 1e-4))
+    _table_gradients_match(p, d, cap, f"{n} points")
+
+
 def test_records_crowd_one_bin():
     """Points chosen so that, at the finest level, at least three of their four vertices fall into the
     first of four slot ranges: the tile's records are all distinct (the workgroup streams them sorted
