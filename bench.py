@@ -10,20 +10,25 @@ every input already resident in HBM.  Prints ONE JSON line:
                duration, measured with events on the launch stream inside the timed loop
   cpu_baseline the CPU oracle (a scalar-code OpenMP port of the reference kernels) timed on this
                machine's host cores on a bounded sample of the same workload
-  probes       measured streaming / random-gather / random-atomic rates of this GPU
+  probes       measured streaming / random-gather / random-atomic rates of this GPU; the gather probe is
+               swept over loads in flight per lane, workgroup size and load flavour, and the fastest
+               setting found is the rate the gathers are priced at
   measured_roofline
                per phase, a lower bound of the phase's time built from measurements of this GPU in
-               this run: the slots every level really touches are replayed through a gather-only
-               probe (minus the same probe with all slots equal, which keeps its streaming but takes
-               the gathers out), next to the time to stream the phase's compulsory bytes at the copy
-               probe's rate and the time to issue the kernels' vector instructions; frac = bound /
-               measured, at most 1
+               this run, with no term that depends on how the kernels are written: the slots every
+               level really touches are replayed through the gather-only probe (its default and its
+               fastest setting, whichever is quicker at that level, minus the same probe with all
+               slots equal, which keeps its streaming but takes the gathers out), next to the time to
+               stream the phase's compulsory bytes at the copy probe's rate; frac = bound / measured,
+               at most 1.  `with_vector_issue` repeats it with the time to issue the kernels' own
+               vector instructions as a third term: a diagnostic, not a bound of the problem
   hbm_traffic_rate
                HBM bytes per launch from hardware counters (profiles/hbm_traffic.json) / phase time
 
 Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu]
 """
 import argparse
+import itertools
 import json
 import os
 import sys
@@ -47,6 +52,24 @@ def kernel_source_digest():
         with open(os.path.join(csrc, name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]
+
+
+def traffic_entry_matches(entry, kernels, second_order):
+    """Whether a phase's entry of profiles/hbm_traffic.json was summed over exactly the kernels the phase
+    launches (by name, the scattering kernel also by its second-order template argument) and its totals
+    are the sums of its per-kernel rows."""
+    rows = entry.get("per_kernel")
+    if not isinstance(rows, dict) or sorted(rows) != sorted(entry.get("kernels", [])):
+        return False
+    if sorted(k.split("<")[0] for k in rows) != sorted(kernels):
+        return False
+    for k in rows:
+        if k.startswith("backward_table_kernel<"):
+            args = [a.strip() for a in k[k.index("<") + 1:k.rindex(">")].split(",")]
+            if len(args) < 3 or (args[2] == "true") != second_order:
+                return False
+    total = sum(r["hbm_bytes"] for r in rows.values())
+    return abs(total - entry["hbm_bytes"]) <= 1e-6 * max(total, 1.0)
 
 
 def algorithmic_bytes(w):
@@ -168,17 +191,44 @@ def run_probes(torch, capacity, n_threads, per_thread):
     out = torch.empty(n_threads * 2, dtype=torch.float32, device=dev)
     t = _timed(torch, lambda: lib.penc_probe_gather(table.data_ptr(), idx.data_ptr(), n_threads, per_thread, out.data_ptr(), st()))
     res["gather_Gacc_per_s"] = n_threads * per_thread / t / 1e9
+    # Is that probe a ceiling?  The same gathers with 1, 2 or 4 points per lane (K, 2K, 4K loads in flight),
+    # workgroups of 64 to 1024 threads, and ordinary, non-temporal and raw-buffer loads with each cache policy.
+    sweep = []
+    if per_thread in GATHER_VARIANT_K and n_threads % 4 == 0:
+        for points, block, kind in itertools.product((1, 2, 4), (64, 256, 1024), sorted(GATHER_LOAD_KINDS)):
+            call = lambda: lib.penc_probe_gather_variant(table.data_ptr(), capacity, idx.data_ptr(), n_threads, per_thread, points,
+                                                         block, kind, out.data_ptr(), st())
+            assert call() == 0
+            sweep.append((_timed(torch, call, iters=10, warm=2), points, block, kind))
+        sweep.sort()
+        best = sweep[0]
+        res["gather_sweep"] = {
+            "best_Gacc_per_s": n_threads * per_thread / best[0] / 1e9,
+            "best": {"points_per_lane": best[1], "block_threads": best[2], "load": GATHER_LOAD_KINDS[best[3]]},
+            "worst_Gacc_per_s": n_threads * per_thread / sweep[-1][0] / 1e9,
+            "best_per_load_Gacc_per_s": {GATHER_LOAD_KINDS[k]: n_threads * per_thread / min(t for t, _, _, kk in sweep if kk == k) / 1e9
+                                          for k in sorted(GATHER_LOAD_KINDS)},
+            "settings_tried": len(sweep),
+        }
+        res["gather_best_variant"] = list(best[1:])
     t = _timed(torch, lambda: lib.penc_probe_scatter(table.data_ptr(), idx.data_ptr(), n_threads, per_thread, st()))
     res["scatter_Gatomic_per_s"] = 2 * n_threads * per_thread / t / 1e9
     res["slice_bytes"] = capacity * 8
     return res
 
 
-def gather_pattern_seconds(torch, native, w, fp, table, pos):
+GATHER_VARIANT_K = (4, 5, 9)  # gathers per point the variant probe is built for (pos_dim 3, 4 and 8)
+GATHER_LOAD_KINDS = {0: "global_load", 1: "global_load nt (compiler's non-temporal)", 2: "buffer_load", 3: "buffer_load sc0",
+                     4: "buffer_load nt", 18: "buffer_load sc1", 19: "buffer_load sc0 sc1"}
+
+
+def gather_pattern_seconds(torch, native, w, fp, table, pos, variant=None):
     """Per level: what the D+1 gathers per point cost on this memory system for the slots the workload
     really touches.  The slots (penc_simplex_debug, the forward's own device routine) are replayed
     through the gather-only probe; the same probe with every slot equal to 0 has the same streaming
-    traffic (index reads, one store per point) but cache-resident gathers, and is subtracted."""
+    traffic (index reads, one store per point) but cache-resident gathers, and is subtracted.  With
+    `variant` (points per lane, workgroup size, load flavour: the fastest setting of the sweep) every
+    level is replayed through that setting as well and the quicker of the two counts."""
     from permutohedral_encoding_amd import probes
     lib, plib = native.lib(), probes.lib()
     st = torch.cuda.current_stream().cuda_stream
@@ -187,6 +237,11 @@ def gather_pattern_seconds(torch, native, w, fp, table, pos):
     zeros = torch.zeros((d + 1, n), dtype=torch.int32, device="cuda")
     level_table = table[0]
     t_zero = _timed(torch, lambda: plib.penc_probe_gather(level_table.data_ptr(), zeros.data_ptr(), n, d + 1, out.data_ptr(), st), iters=10)
+    t_zero_variant = None
+    if variant is not None:
+        run_variant = lambda idx_: plib.penc_probe_gather_variant(level_table.data_ptr(), cap, idx_.data_ptr(), n, d + 1, variant[0],
+                                                                  variant[1], variant[2], out.data_ptr(), st)
+        t_zero_variant = _timed(torch, lambda: run_variant(zeros), iters=10)
     slot = torch.empty((1, n, d + 1), dtype=torch.int32, device="cuda")
     result = []
     for l in range(levels):
@@ -197,7 +252,10 @@ def gather_pattern_seconds(torch, native, w, fp, table, pos):
         idx = slot[0].t().contiguous()
         level_table = table[l]
         t_real = _timed(torch, lambda: plib.penc_probe_gather(level_table.data_ptr(), idx.data_ptr(), n, d + 1, out.data_ptr(), st), iters=10)
-        result.append(max(t_real - t_zero, 0.0))
+        cost = max(t_real - t_zero, 0.0)
+        if variant is not None:
+            cost = min(cost, max(_timed(torch, lambda: run_variant(idx), iters=10) - t_zero_variant, 0.0))
+        result.append(cost)
     return result, t_zero
 
 
@@ -205,8 +263,10 @@ VALU_WAVE_INSTR_PER_S = 256 * 4 * 2.4e9 / 4  # 256 CUs x 4 SIMDs, one wave64 vec
 
 
 def measured_roofline(w, phases, window, gather_s, copy_GBps, valu_per_point_level):
-    """Lower bound per phase = sum over levels of max(gather pattern, compulsory streaming, vector issue).
-    Every term is a lower bound of what the level costs, so the sum is one for the phase."""
+    """Lower bound per phase = sum over levels of max(gather pattern, compulsory streaming).  Both terms
+    are properties of the problem on this memory system, so the sum is a bound for any implementation.
+    With `valu_per_point_level` (the shipped kernels' own instruction counts) the time to issue those
+    instructions is a third term: that figure describes the kernels, not the problem."""
     d, l, c, n = w.pos_dim, w.nr_levels, w.capacity, w.nr_points
     copy = copy_GBps * 1e9
     pos_bytes = 4.0 * d * n / l
@@ -340,10 +400,12 @@ def main():
     phase_bytes["double_backward"] = ab["double_backward"]
     # tables with more than 64 slot ranges of 8192 slots are reduced by workgroups that walk several levels
     reducer = "bin_reduce_levels_kernel" if w.capacity > 64 * 8192 else "bin_reduce_kernel"
-    kernel_names = {"forward": "forward_kernel",
-                    "backward": "+".join((["fill_zero_kernel", "backward_table_kernel", reducer] if want_table else [])
-                                         + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else [])),
-                    "double_backward": "grad_grad_kernel+fill_zero_kernel+backward_table_kernel<second order>+" + reducer}
+    phase_kernels = {"forward": ["forward_kernel"],
+                     "backward": (["fill_zero_kernel", "backward_table_kernel", reducer] if want_table else [])
+                                 + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else []),
+                     "double_backward": ["grad_grad_kernel", "fill_zero_kernel", "backward_table_kernel", reducer]}
+    kernel_names = {k: "+".join(v) for k, v in phase_kernels.items()}
+    kernel_names["double_backward"] = kernel_names["double_backward"].replace("backward_table_kernel", "backward_table_kernel<second order>")
     dominant = max(phase_ms, key=phase_ms.get)
     achieved = phase_bytes[dominant] * w.point_levels / (phase_ms[dominant] * 1e-3) / 1e9
     # HBM bytes per launch and vector instructions per point-level come from the committed counter
@@ -363,10 +425,12 @@ def main():
         recorded = recorded.get(w.name, {})
         for name in phase_ms:
             entry = recorded.get(name)
-            if entry and entry.get("kernels") == kernel_names[name]:
+            if entry and traffic_entry_matches(entry, phase_kernels[name], second_order=name == "double_backward"):
                 per_phase[name] = entry["hbm_bytes"]
                 if entry.get("valu_wave_instr"):
                     valu_per_point_level[name] = entry["valu_wave_instr"] * 64.0 / w.point_levels
+            elif entry:
+                traffic_note += f"; the entry for {name} does not cover the kernels this phase launches: not used"
     roofline = {"bound": "hbm", "kernel": kernel_names[dominant], "achieved": achieved, "peak": HBM_PEAK_GBPS,
                 "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": per_phase.get(dominant),
                 "traffic_source": traffic_note,
@@ -398,19 +462,30 @@ def main():
     if not args.no_probes:
         result["probes"] = run_probes(torch, cap, n, d + 1)
         pr = result["probes"]
-        gather_s, t_zero = gather_pattern_seconds(torch, _native, w, fp, inp.m_lattice_values, inp.m_positions_raw)
-        bound_ms = measured_roofline(w, phases, inputs["window"], gather_s, pr["copy_GBps"], valu_per_point_level)
+        gather_s, t_zero = gather_pattern_seconds(torch, _native, w, fp, inp.m_lattice_values, inp.m_positions_raw,
+                                                  pr.pop("gather_best_variant", None))
+        bound_ms = measured_roofline(w, phases, inputs["window"], gather_s, pr["copy_GBps"], {})
         result["measured_roofline"] = {
             "bound_ms": bound_ms,
             "frac": {k: bound_ms[k] / phase_ms[k] for k in bound_ms},
             "step_bound_ms": sum(bound_ms.values()),
             "step_frac": sum(bound_ms.values()) / sum(phase_ms.values()),
             "gather_pattern_us_per_level": [round(x * 1e6, 2) for x in gather_s],
-            "note": "per level max(replay of the level's own slots through the gather-only probe minus the same "
-                    "probe with all slots equal, compulsory bytes at the copy probe's rate, vector instructions at "
-                    "one per 4 clocks per SIMD), summed over the levels; a table gradient or second table pass "
-                    "counts its slot accesses like gathers; frac = bound / measured phase time",
+            "note": "per level max(replay of the level's own slots through the gather-only probe, at its default or at the "
+                    "fastest setting of the sweep, minus the same probe with all slots equal; compulsory bytes at the copy "
+                    "probe's rate), summed over the levels; a table gradient or second table pass counts its slot accesses "
+                    "like gathers; frac = bound / measured phase time",
         }
+        if valu_per_point_level:
+            with_valu = measured_roofline(w, phases, inputs["window"], gather_s, pr["copy_GBps"], valu_per_point_level)
+            result["measured_roofline"]["with_vector_issue"] = {
+                "bound_ms": with_valu,
+                "frac": {k: with_valu[k] / phase_ms[k] for k in with_valu},
+                "step_frac": sum(with_valu.values()) / sum(phase_ms.values()),
+                "note": "the same with a third term per level: the shipped kernels' own vector instructions (hardware counter) at "
+                        "one per 4 clocks per SIMD.  It describes the kernels, not the problem: a kernel that issues more "
+                        "instructions raises it.  Diagnostic only.",
+            }
         if per_phase:
             result["hbm_traffic_rate"] = {
                 "GBps": {k: per_phase[k] / (phase_ms[k] * 1e-3) / 1e9 for k in phase_ms if k in per_phase},

@@ -11,6 +11,12 @@
  *            writes one 8-byte result; idx holds per_thread * n_threads slots.  Fed with the slots a
  *            workload really uses (penc_simplex_debug), level by level, it measures what the gathers of
  *            that level cost on this memory system.
+ *   gather_variant : the same gathers with the knobs a kernel author could turn: `points_per_thread`
+ *            (1, 2 or 4: per_thread * points_per_thread loads are in flight per lane; per_thread is 4, 5 or 9),
+ *            `block_threads` (a multiple of 64 up to 1024) and `load_kind` (0 ordinary global load, 1 the
+ *            compiler's non-temporal load, 2 + bits a raw buffer load with cache-policy bits: 1 = sc0, 2 = nt,
+ *            16 = sc1; accepted: 2, 3, 4, 18, 19).  n_threads must be a multiple of points_per_thread.  The
+ *            benchmark sweeps them and prices the encoding's gathers at the fastest setting found.
  *   scatter: every thread issues `per_thread` pairs of fp32 atomic adds at table[idx[k][thread]]
  */
 #ifndef PENC_PROBES_H_
@@ -25,6 +31,9 @@ extern "C" {
 int penc_probe_copy(const float* src, float* dst, int64_t n_float4, void* stream);
 int penc_probe_gather(const float* table, const int* idx, int64_t n_threads, int per_thread,
                       float* out, void* stream);
+int penc_probe_gather_variant(const float* table, int64_t table_slots, const int* idx, int64_t n_threads,
+                              int per_thread, int points_per_thread, int block_threads, int load_kind,
+                              float* out, void* stream);
 int penc_probe_scatter(float* table, const int* idx, int64_t n_threads, int per_thread, void* stream);
 
 #ifdef __cplusplus

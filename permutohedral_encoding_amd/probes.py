@@ -11,6 +11,8 @@ _p = ctypes.c_void_p
 _SIGNATURES = {
     "penc_probe_copy": (ctypes.c_int, [_p, _p, ctypes.c_int64, _p]),
     "penc_probe_gather": (ctypes.c_int, [_p, _p, ctypes.c_int64, ctypes.c_int, _p, _p]),
+    "penc_probe_gather_variant": (ctypes.c_int, [_p, ctypes.c_int64, _p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                ctypes.c_int, _p, _p]),
     "penc_probe_scatter": (ctypes.c_int, [_p, _p, ctypes.c_int64, ctypes.c_int, _p]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

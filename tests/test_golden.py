@@ -47,10 +47,13 @@ def test_hip_matches_golden(d):
     cap = c["table"].shape[1]
     enc, fp = make_encoding(d, c["sigmas"], c["shift"])
     assert np.array_equal(fp.m_scale_factor.cpu().numpy(), c["sf"])
-    dbg = enc.simplex_debug(to_gpu(c["pos"]), cap)
-    for k in ("rem0", "rank", "slot"):
-        assert np.array_equal(dbg[k].cpu().numpy(), c[k]), k
-    assert np.array_equal(dbg["barycentric"].cpu().numpy(), c["bary"])
+    # both device routines that produce slots and weights: the select chains of the scattering and
+    # position-gradient kernels, and the LDS rank sort of the forward and grad-of-grad kernels
+    for gather_path in (False, True):
+        dbg = enc.simplex_debug(to_gpu(c["pos"]), cap, gather_path=gather_path)
+        for k in ("rem0", "rank", "slot"):
+            assert np.array_equal(dbg[k].cpu().numpy(), c[k]), (k, gather_path)
+        assert np.array_equal(dbg["barycentric"].cpu().numpy(), c["bary"]), gather_path
     inp = _native.EncodingInput(to_gpu(c["table"]), to_gpu(c["pos"]), to_gpu(c["window"]), True, True)
     out = enc.forward(inp).cpu().numpy()
     assert np.all(np.abs(out - c["out"]) <= 1e-6 + 1e-5 * np.abs(c["out"]))

@@ -859,3 +859,74 @@ def test_large_size_identities_in_the_other_dimensions(d):
         _native.LEVELS_PER_PASS = saved
     assert torch.allclose(tg, tg_direct, rtol=1e-3, atol=1e-5 * tg.abs().max().item())
     assert torch.allclose(tg2, tg2_direct, rtol=1e-3, atol=1e-5 * tg2.abs().max().item())
+
+
+# ----------------------------------------------------------------------------- randomized geometries
+
+def _random_geometry(seed):
+    """Input dimension, features, capacity (powers of two and not, from a thousand slots to beyond 2^22),
+    number of points and levels, scale range, masked level and workspace size, all drawn from `seed`."""
+    rng = np.random.default_rng(1000 + seed)
+    d = int(rng.integers(2, 9))
+    feat = int(rng.choice([2, 2, 4, 8]))
+    kind = int(rng.integers(0, 4))
+    if kind == 0:
+        cap = int(rng.integers(1 << 10, 1 << 19))
+    elif kind == 1:
+        cap = int(rng.integers(1 << 19, 1 << 22))
+    elif kind == 2:
+        cap = int(rng.integers(1 << 22, 1 << 23))
+    else:
+        cap = 1 << int(rng.integers(12, 24))
+    cap = min(cap, ((1 << 31) - 1) // (feat * 6))
+    n = int(rng.integers(1000, 200000))
+    levels = int(rng.integers(1, 6))
+    while levels > 1 and cap * feat * levels > 1 << 27:  # keeps the oracle's fp64 sums of the table gradient within a few GB
+        levels -= 1
+    sigma_lo = float(10 ** rng.uniform(-3.5, -1.0))
+    masked = int(rng.integers(levels)) if levels > 2 and rng.random() < 0.4 else None
+    workspace = ["full", "full", "third", "none"][int(rng.integers(0, 4))]
+    return dict(d=d, feat=feat, cap=cap, n=n, levels=levels, sigma_lo=sigma_lo, masked=masked, workspace=workspace,
+                problem_seed=int(rng.integers(1 << 30)))
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_geometry_all_phases_match_oracle(seed, monkeypatch):
+    """Twenty seeded random problems through every phase against the oracle.  Run under -x the suite
+    stops at the first geometry that disagrees; the assertion message names it."""
+    from permutohedral_encoding_amd import _native
+    g = _random_geometry(seed)
+    d, feat, cap, n, levels = g["d"], g["feat"], g["cap"], g["n"], g["levels"]
+    what = f"seed {seed}: {g}"
+    p = random_problem(d, n, levels, 1, seed=g["problem_seed"], sigma_range=(1.0, g["sigma_lo"]), nr_feat=feat)
+    if g["masked"] is not None:
+        p["window"][g["masked"]] = 0.0
+    p["table"] = np.random.default_rng(g["problem_seed"] + 1).uniform(-1, 1, (levels, cap, feat)).astype(np.float32)
+    sf = orc.scale_factors(d, p["sigmas"])
+    if g["workspace"] == "none":
+        monkeypatch.setattr(_native, "MAX_WORKSPACE_BYTES", 0)
+    elif g["workspace"] == "third":
+        full = int(_native.lib().penc_scatter_workspace_bytes(d, n, levels * feat // 2, cap, 0))
+        monkeypatch.setattr(_native, "MAX_WORKSPACE_BYTES", max(full // 3, 1 << 16))
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
+    inp = gpu_input(p)
+
+    want = orc.simplex(p["pos"], sf, p["shift"], cap)
+    for gather_path in (False, True):
+        dbg = enc.simplex_debug(to_gpu(p["pos"]), cap, gather_path=gather_path)
+        assert np.array_equal(dbg["slot"].cpu().numpy(), want["slot"]), what
+        assert np.array_equal(dbg["rank"].cpu().numpy(), want["rank"]), what
+        del dbg
+    out = enc.forward(inp).cpu().numpy()
+    assert np.array_equal(out, orc.forward(p["pos"], p["table"], sf, p["shift"], p["window"])), what
+
+    tg, pg = enc.backward(inp, to_gpu(p["grad"]))
+    wt = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
+    assert_sum_close(tg.cpu().numpy(), wt["grad64"], wt["abs64"], SUM_RTOL, f"table gradient, {what}")
+    check_pos_grad(pg.cpu().numpy(), orc.backward_pos(p["pos"], p["table"], sf, p["shift"], p["window"], p["grad"]))
+    del tg, pg, wt
+
+    tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(p["dpos"]), to_gpu(p["grad"]))
+    wd = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
+    assert_sum_close(tg2.cpu().numpy(), wd["grad64"], wd["abs64"], SUM_RTOL, f"second-order table gradient, {what}")
+    check_grad_grad(ggs.cpu().numpy(), wd)

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(probes.LIB_PATH)
     for n in probe_names:
         assert hasattr(handle, n), f"{n} is declared in include/penc_probes.h but not exported"
-    assert set(probe_names) == set(probes.EXPORTED_SYMBOLS) and len(probe_names) == 3
+    assert set(probe_names) == set(probes.EXPORTED_SYMBOLS) and len(probe_names) == 4
 
 
 def test_status_strings_and_extra_levels():
@@ -225,3 +225,63 @@ def test_workspace_request_is_capped_and_shrinks_when_memory_runs_out(monkeypatc
     with pytest.raises(torch.cuda.OutOfMemoryError):
         _native.scatter_workspace(d, n, levels, cap, "cpu", positions_grad=True, fixed_bytes=1000, required_bytes=1000)
     assert requests[-1] == 1000
+
+
+def _counter_rows(workload):
+    """(phase, kernel) -> (memory-side bytes, vector instructions) from the table of profiles/<workload>_counters.md."""
+    rows = {}
+    header = None
+    for line in open(os.path.join(ROOT, "profiles", f"{workload}_counters.md")):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if line.startswith("| phase | kernel | avg us"):
+            header = cells
+        elif header and line.startswith("|") and not line.startswith("|---") and len(cells) == len(header):
+            r = dict(zip(header, cells))
+            mib = float(r["memory-side read MiB"]) + float(r["memory-side written MiB"])
+            rows[(r["phase"], r["kernel"].strip("`"))] = (mib * 2 ** 20, float(r["VALU instr (wave)"]))
+        elif header and not line.startswith("|"):
+            header = None
+    return rows
+
+
+@pytest.mark.parametrize("workload", ["c2", "c3", "c4", "c5"])
+def test_traffic_summary_is_the_sum_of_the_counter_rows_it_names(workload):
+    """profiles/hbm_traffic.json (what bench.py reads) against the per-kernel tables beside it: every
+    phase's bytes and vector instructions are the sums of the rows of the kernels the phase names, every
+    kernel the phase launches is named, and the scattering kernel of each phase is the right instance."""
+    import json
+    import bench
+    recorded = json.load(open(os.path.join(ROOT, "profiles", "hbm_traffic.json")))
+    assert workload in recorded
+    w = workloads.WORKLOADS[workload]
+    want_table, want_pos = "backward_table" in w.phases, "backward_pos" in w.phases
+    reducer = "bin_reduce_levels_kernel" if w.capacity > 64 * 8192 else "bin_reduce_kernel"
+    expected = {"forward": ["forward_kernel"]}
+    if want_table or want_pos:
+        expected["backward"] = ((["fill_zero_kernel", "backward_table_kernel", reducer] if want_table else [])
+                                + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else []))
+    if "double_backward" in w.phases:
+        expected["double_backward"] = ["grad_grad_kernel", "fill_zero_kernel", "backward_table_kernel", reducer]
+    rows = _counter_rows(workload)
+    assert sorted(recorded[workload]) == sorted(expected)
+    for phase, kernels in expected.items():
+        entry = recorded[workload][phase]
+        assert bench.traffic_entry_matches(entry, kernels, second_order=phase == "double_backward"), (phase, entry["kernels"])
+        table_bytes = sum(rows[(phase, k)][0] for k in entry["kernels"])
+        table_valu = sum(rows[(phase, k)][1] for k in entry["kernels"])
+        # the tables are rounded to 0.1 MiB and three significant digits per row
+        assert abs(entry["hbm_bytes"] - table_bytes) <= 0.11 * 2 ** 20 * len(entry["kernels"]), phase
+        assert abs(entry["valu_wave_instr"] - table_valu) <= 0.006 * table_valu + 1, phase
+    # a wrongly attributed entry is refused: the first-order scatter does not serve the double backward
+    if "double_backward" in expected and "backward_table_kernel" in expected.get("backward", []):
+        assert not bench.traffic_entry_matches(recorded[workload]["backward"], expected["double_backward"], second_order=True)
+
+
+def test_profile_summary_attributes_shared_kernels_by_dispatch_order():
+    from permutohedral_encoding_amd import profile_summary as ps
+    k = ["forward_kernel<4, 2, float>", "backward_pos_kernel<4, 2, float>", "reduce_level_groups_kernel",
+         "grad_grad_kernel<4, 2, float>", "fill_zero_kernel", "backward_table_kernel<4, false, true, false>", "bin_reduce_kernel<true>",
+         "fill_zero_kernel", "backward_table_kernel<4, false, false, false>", "bin_reduce_kernel<true>", "at::native::copy_kernel", "copy_kernel"]
+    assert ps.phase_of_dispatches(k) == ["forward", "backward", "backward", "double_backward", "double_backward", "double_backward",
+                                         "double_backward", "backward", "backward", "backward", None, None]
+    assert ps.short("void penc::backward_table_kernel<3, false, true, false>(int, int)") == "backward_table_kernel<3, false, true, false>"
