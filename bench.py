@@ -158,6 +158,43 @@ def module_level(torch, w, inputs, steps, warmup):
     return {"ms_per_step": ms, "point_levels_per_s": w.point_levels / (ms * 1e-3), "what": what}
 
 
+def optimizer_leg(torch, lib, w, table, tgrad, touched, run_gradients, clear_touched):
+    """The optimizer step on the workload's table after its gradient calls: torch.optim.AdamW (every entry of
+    the table, several kernels), penc_adamw_step with skip_zero_gradients (one kernel that reads the whole
+    gradient) and penc_adamw_step_sparse (the slot ranges the gradient calls marked, nothing else).  Each is
+    timed alone, on the gradient one step leaves; the sparse one is re-armed by repeating the gradient calls
+    outside its timing.  Not part of `value`."""
+    from permutohedral_encoding_amd.optim import AdamW
+    st = torch.cuda.current_stream().cuda_stream
+    kw = dict(lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0)
+    res = {}
+    run_gradients()
+    dense_grad = tgrad.clone()
+    for name, make in (("torch_adamw_ms", lambda p: torch.optim.AdamW([p], **kw)),
+                       ("fused_adamw_skip_zero_ms", lambda p: AdamW([p], skip_zero_gradients=True, **kw))):
+        p = torch.nn.Parameter(table.clone())
+        p.grad = dense_grad
+        opt = make(p)
+        res[name] = _timed(torch, opt.step, iters=5, warm=2) * 1e3
+        del opt, p
+    p, m, v = table.clone(), torch.zeros_like(table), torch.zeros_like(table)
+    times = []
+    for k in range(6):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        rc = lib.penc_adamw_step_sparse(p.data_ptr(), tgrad.data_ptr(), m.data_ptr(), v.data_ptr(), 2, w.nr_levels, w.capacity,
+                                        touched.data_ptr(), 1e-3, 0.9, 0.999, 1e-8, 0.0, k + 1, 1, st)
+        e1.record()
+        assert rc == 0, rc
+        torch.cuda.synchronize()
+        times.append(e0.elapsed_time(e1))
+        run_gradients()
+    clear_touched()
+    res["sparse_adamw_ms"] = float(np.median(times[1:]))
+    res["touched_fraction_of_slot_ranges"] = None
+    return res
+
+
 def _timed(torch, fn, iters=20, warm=3):
     for _ in range(warm):
         fn()
@@ -272,6 +309,9 @@ def measured_roofline(w, phases, window, gather_s, copy_GBps, valu_per_point_lev
     pos_bytes = 4.0 * d * n / l
     out = {}
     for name, _ in phases:
+        if name == "clear_touched":  # bookkeeping of the sparse table gradient: no bound of its own
+            out[name] = 0.0
+            continue
         # (slot-access passes over the table, streamed bytes per level) of the phase
         if name == "forward":
             passes, stream = 1, 8.0 * n + pos_bytes
@@ -307,6 +347,12 @@ def main():
     ap.add_argument("--levels-per-pass", type=int, default=0,
                     help="levels binned per scatter pass (0: library default, -1: no workspace, direct atomics)")
     ap.add_argument("--cpu-sample", type=int, default=1 << 20, help="points in the CPU baseline sample")
+    ap.add_argument("--sparse-table-grad", action="store_true",
+                    help="table gradients through the sparse entry points: both gradient calls add into one array kept across "
+                         "steps and mark the slot ranges they touch, and the step ends by clearing what was touched "
+                         "(penc_clear_touched) instead of each call clearing a dense gradient first")
+    ap.add_argument("--optimizer", action="store_true",
+                    help="with --sparse-table-grad: also time the optimizer step on the table (torch AdamW, fused, sparse)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on one GPU only; --gpus N with N > 1 is not supported", file=sys.stderr)
@@ -353,15 +399,34 @@ def main():
                        int(lib.penc_positions_workspace_bytes(d, n, levels)))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
 
+    sparse = args.sparse_table_grad and (want_table or want_double)
+    touched = None
+    if sparse:
+        tgrad.zero_()
+        touched = torch.zeros(int(lib.penc_touched_map_entries(2, levels, cap)), dtype=torch.int32, device=dev)
+
     def backward():
-        rc = lib.penc_backward(d, 2, n, levels, cap, P(inp.m_positions_raw), P(inp.m_lattice_values), P(sf), P(shift),
-                               P(win), P(grad), P(tgrad) if want_table else None, P(pgrad), P(ws), ws_bytes, stream)
+        if sparse and want_table:
+            rc = lib.penc_backward_sparse(d, 2, n, levels, cap, P(inp.m_positions_raw), P(inp.m_lattice_values), P(sf), P(shift),
+                                          P(win), P(grad), 0, P(tgrad), P(touched), P(pgrad), P(ws), ws_bytes, stream)
+        else:
+            rc = lib.penc_backward(d, 2, n, levels, cap, P(inp.m_positions_raw), P(inp.m_lattice_values), P(sf), P(shift),
+                                   P(win), P(grad), P(tgrad) if want_table else None, P(pgrad), P(ws), ws_bytes, stream)
         assert rc == 0, rc
 
     def double_backward():
-        rc = lib.penc_double_backward_from_positions(d, 2, n, levels, cap, P(inp.m_positions_raw),
-                                                     P(inp.m_lattice_values), P(sf), P(shift), P(win), P(dpos), P(grad),
-                                                     P(tgrad), P(ggs), 0, P(ws), ws_bytes, stream)
+        if sparse:
+            rc = lib.penc_double_backward_from_positions_sparse(d, 2, n, levels, cap, P(inp.m_positions_raw),
+                                                                P(inp.m_lattice_values), P(sf), P(shift), P(win), P(dpos),
+                                                                P(grad), 0, P(tgrad), P(touched), P(ggs), 0, P(ws), ws_bytes, stream)
+        else:
+            rc = lib.penc_double_backward_from_positions(d, 2, n, levels, cap, P(inp.m_positions_raw),
+                                                         P(inp.m_lattice_values), P(sf), P(shift), P(win), P(dpos), P(grad),
+                                                         P(tgrad), P(ggs), 0, P(ws), ws_bytes, stream)
+        assert rc == 0, rc
+
+    def clear_touched():
+        rc = lib.penc_clear_touched(P(tgrad), 2, levels, cap, P(touched), stream)
         assert rc == 0, rc
 
     phases = [("forward", forward)]
@@ -369,6 +434,8 @@ def main():
         phases.append(("backward", backward))
     if want_double:
         phases.append(("double_backward", double_backward))
+    if sparse:
+        phases.append(("clear_touched", clear_touched))
 
     for _ in range(args.warmup):
         for _, fn in phases:
@@ -398,12 +465,17 @@ def main():
     phase_bytes = {"forward": ab["forward"]}
     phase_bytes["backward"] = (ab["backward_table"] if want_table else 0.0) + (ab["backward_pos"] if want_pos else 0.0)
     phase_bytes["double_backward"] = ab["double_backward"]
+    phase_bytes["clear_touched"] = 0.0  # bookkeeping of the sparse table gradient: no algorithmic bytes of its own
     # tables with more than 64 slot ranges of 8192 slots are reduced by workgroups that walk several levels
     reducer = "bin_reduce_levels_kernel" if w.capacity > 64 * 8192 else "bin_reduce_kernel"
     phase_kernels = {"forward": ["forward_kernel"],
                      "backward": (["fill_zero_kernel", "backward_table_kernel", reducer] if want_table else [])
                                  + (["backward_pos_kernel", "reduce_level_groups_kernel"] if want_pos else []),
                      "double_backward": ["grad_grad_kernel", "fill_zero_kernel", "backward_table_kernel", reducer]}
+    phase_kernels["clear_touched"] = ["touched_ranges_kernel"]
+    if sparse:  # nothing is cleared before the scatter
+        for name in ("backward", "double_backward"):
+            phase_kernels[name] = [k for k in phase_kernels[name] if k != "fill_zero_kernel"]
     kernel_names = {k: "+".join(v) for k, v in phase_kernels.items()}
     kernel_names["double_backward"] = kernel_names["double_backward"].replace("backward_table_kernel", "backward_table_kernel<second order>")
     dominant = max(phase_ms, key=phase_ms.get)
@@ -451,7 +523,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"{w.name}: pos_dim={d} levels={levels} capacity=2^{cap.bit_length() - 1} feat=2 "
-                               f"points=2^{n.bit_length() - 1} phases={'+'.join(p for p, _ in phases)}"},
+                               f"points=2^{n.bit_length() - 1} phases={'+'.join(p for p, _ in phases)}"
+                               + (" (sparse table gradient)" if sparse else "")},
         "phases_ms": phase_ms,
         "phases_ms_median": phase_median,
         "phases_ms_min": phase_min,
@@ -492,6 +565,16 @@ def main():
                 "copy_probe_GBps": pr["copy_GBps"],
                 "note": "HBM bytes per launch from hardware counters (profiles/) / measured phase time",
             }
+    if sparse and args.optimizer:
+        def run_gradients():
+            for name, fn in phases:
+                if name in ("backward", "double_backward"):
+                    fn()
+        run_gradients()
+        marked = float((touched != 0).float().mean().item())
+        clear_touched()
+        result["optimizer_step"] = optimizer_leg(torch, lib, w, inp.m_lattice_values, tgrad, touched, run_gradients, clear_touched)
+        result["optimizer_step"]["touched_fraction_of_slot_ranges"] = marked
     if not args.no_module:
         result["module_level"] = module_level(torch, w, inputs, args.steps, args.warmup)
     if not args.no_cpu:

@@ -230,6 +230,43 @@ int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* ex
                     double beta1, double beta2, double eps, double weight_decay, int64_t step, int skip_zero_gradients,
                     void* stream);
 
+/* The table gradient for tables that dwarf the batch: the caller keeps ONE gradient array and a map of
+ * the slot ranges that hold anything across calls, and no call touches more of either than the batch does.
+ *   touched  uint32 [L * F/2][R], R = ceil(capacity / penc_touched_range_slots(capacity)) slot ranges per level
+ *            and pair of features (penc_touched_map_entries() entries in all): nonzero where the gradient
+ *            may be nonzero.
+ * Contract: wherever `touched` is 0 the gradient is 0 (both start zeroed by the caller; penc_clear_touched and
+ * penc_adamw_step_sparse restore that state).  penc_backward_sparse and
+ * penc_double_backward_from_positions_sparse then ADD their sums into lattice_values_grad (so the two calls of a
+ * training step accumulate into the one array, which is what autograd would do with a second dense add) and mark
+ * the ranges they reached; they clear nothing.  Everything else is as in penc_backward /
+ * penc_backward_rowmajor (grad_row_stride 0 or a row stride) and penc_double_backward_from_positions.
+ * penc_adamw_step_sparse applies penc_adamw_step with skip_zero_gradients to the touched ranges only and, with
+ * `clear`, zeroes the gradients it used and the map; penc_clear_touched only does the clearing.  Both cost one
+ * workgroup per (range, level) that leaves at once where nothing was added: the step on a 2^22-slot, 24-level
+ * table follows what the batch touched instead of reading 768 MiB of gradient.
+ * Replaces: the `zeros` of the whole gradient in every call (src/Encoding.cu:141, 246), autograd's dense
+ * accumulation of the two table gradients, and the full-table optimizer step of the reference's training
+ * protocol (examples/performance.py:99-101). */
+size_t penc_touched_map_entries(int nr_feat, int nr_levels, int capacity);
+int penc_touched_range_slots(int capacity);
+int penc_backward_sparse(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                         const float* positions, const float* lattice_values, const float* scale_factor,
+                         const float* random_shift, const float* anneal_window, const float* grad, int64_t grad_row_stride,
+                         float* lattice_values_grad, uint32_t* touched, float* positions_grad, void* workspace,
+                         size_t workspace_bytes, void* stream);
+int penc_double_backward_from_positions_sparse(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                               const float* positions, const float* lattice_values,
+                                               const float* scale_factor, const float* random_shift,
+                                               const float* anneal_window, const float* double_positions_grad,
+                                               const float* grad, int64_t grad_row_stride, float* lattice_values_grad,
+                                               uint32_t* touched, float* grad_grad_sliced_values, int concat_points,
+                                               void* workspace, size_t workspace_bytes, void* stream);
+int penc_adamw_step_sparse(float* params, float* grads, float* exp_avg, float* exp_avg_sq, int nr_feat, int nr_levels,
+                           int capacity, uint32_t* touched, double lr, double beta1, double beta2, double eps,
+                           double weight_decay, int64_t step, int clear, void* stream);
+int penc_clear_touched(float* grads, int nr_feat, int nr_levels, int capacity, uint32_t* touched, void* stream);
+
 /* dst[c][r] = src[r][c] for a dense row-major rows x cols matrix with cols <= 255 (2 * levels):
  * turns the row-major upstream gradient (N, 2(L+E)) into the grad_sliced_values layout
  * [L+E][2][N] at streaming speed.

@@ -67,6 +67,21 @@ _SIGNATURES = {
     "penc_adamw_step": (ctypes.c_int, [_c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_double, ctypes.c_double,
                                        ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_int64, ctypes.c_int,
                                        ctypes.c_void_p]),
+    "penc_touched_map_entries": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "penc_touched_range_slots": (ctypes.c_int, [ctypes.c_int]),
+    "penc_backward_sparse": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                            _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
+                                            _c_f32p, ctypes.c_void_p, _c_f32p, ctypes.c_void_p, ctypes.c_size_t,
+                                            ctypes.c_void_p]),
+    "penc_double_backward_from_positions_sparse": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+                                                                  ctypes.c_int, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
+                                                                  _c_f32p, _c_f32p, ctypes.c_int64, _c_f32p, ctypes.c_void_p,
+                                                                  _c_f32p, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                                                  ctypes.c_void_p]),
+    "penc_adamw_step_sparse": (ctypes.c_int, [_c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                              ctypes.c_void_p, ctypes.c_double, ctypes.c_double, ctypes.c_double,
+                                              ctypes.c_double, ctypes.c_double, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
+    "penc_clear_touched": (ctypes.c_int, [_c_f32p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]),
     "penc_transpose": (ctypes.c_int, [_c_f32p, _c_f32p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]),
     "penc_simplex_debug": (ctypes.c_int, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _c_f32p, _c_f32p,
                                           _c_f32p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
@@ -215,6 +230,33 @@ def level_major_gradient(grad):
     return grad.contiguous()
 
 
+class SparseTableGrad:
+    """A table gradient kept across calls together with the map of the slot ranges that hold anything
+    (``penc_backward_sparse`` and friends): gradient calls add into ``grad`` and mark ``touched``;
+    ``clear()`` or the sparse optimizer step zero what was touched and nothing else.  No call costs
+    more than the batch touched, whatever the size of the table."""
+
+    def __init__(self, lattice_values):
+        levels, capacity, feat = lattice_values.shape
+        self.nr_levels, self.capacity, self.nr_feat = int(levels), int(capacity), int(feat)
+        self.grad = torch.zeros(lattice_values.shape, dtype=torch.float32, device=lattice_values.device)
+        self.range_slots = int(lib().penc_touched_range_slots(self.capacity))
+        entries = int(lib().penc_touched_map_entries(self.nr_feat, self.nr_levels, self.capacity))
+        self.touched = torch.zeros(entries, dtype=torch.int32, device=lattice_values.device)
+
+    def matches(self, lattice_values):
+        return tuple(self.grad.shape) == tuple(lattice_values.shape) and self.grad.device == lattice_values.device
+
+    def touched_map(self):
+        """(L, F/2, ranges) view of the map: nonzero where a range of ``range_slots`` slots may hold a gradient."""
+        return self.touched.view(self.nr_levels, self.nr_feat // 2, -1)
+
+    def clear(self):
+        with torch.cuda.device(self.grad.device):
+            _check(lib().penc_clear_touched(self.grad.data_ptr(), self.nr_feat, self.nr_levels, self.capacity,
+                                            self.touched.data_ptr(), _stream()), "clear_touched")
+
+
 class EncodingInput:
     """Per-call inputs (reference: ``EncodingInput``, include/permutohedral_encoding/Encoding.cuh:14-29)."""
 
@@ -267,6 +309,15 @@ class EncodingWrapper:
     half_table = None  # set by the module: torch.float16 or torch.bfloat16 to gather from such a copy of the fp32 table
     _half_copy = None
     _half_copy_of = None
+    # set by the module (sparse_table_grad=True): table gradients are added into `sparse_grad`, a SparseTableGrad the
+    # wrapper keeps across calls, and the gradient calls return None for them
+    sparse_table_grad = False
+    sparse_grad = None
+
+    def sparse_grad_for(self, lattice_values):
+        if self.sparse_grad is None or not self.sparse_grad.matches(lattice_values):
+            self.sparse_grad = SparseTableGrad(lattice_values)
+        return self.sparse_grad
 
     def gather_table(self, lattice_values):
         """The tensor the gathering kernels read for ``lattice_values``: the tensor itself, or, with
@@ -350,8 +401,21 @@ class EncodingWrapper:
         grad = grad_sliced_values_monolithic
         self._check_grad(grad, levels, extra, n, allow_rows=True)
         half = lv.dtype in TABLE_FORMATS  # the gradient w.r.t. the table is fp32 either way
-        lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device) if inp.m_require_lattice_values_grad else None
         pos_grad = torch.empty_like(pos) if inp.m_require_positions_grad else None
+        if self.sparse_table_grad and inp.m_require_lattice_values_grad:
+            _require(not half, "sparse_table_grad needs an fp32 table")
+            sparse = self.sparse_grad_for(lv)
+            rows = not grad.is_contiguous()
+            copy_bytes = 4 * self.nr_feat * levels * n + 512 if rows and pos_grad is not None else 0
+            with torch.cuda.device(pos.device):
+                ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, True, pos_grad is not None,
+                                       fixed_bytes=copy_bytes, required_bytes=copy_bytes, nr_feat=self.nr_feat)
+                _check(lib().penc_backward_sparse(
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    _ptr(win), _ptr(grad), grad.stride(2) if rows else 0, _ptr(sparse.grad), _ptr(sparse.touched), _ptr(pos_grad),
+                    _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward_sparse")
+            return None, pos_grad
+        lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device) if inp.m_require_lattice_values_grad else None
         if lv_grad is None and pos_grad is None:
             return None, None
         with torch.cuda.device(pos.device):
@@ -379,10 +443,12 @@ class EncodingWrapper:
                                        _ptr(pos_grad), _ptr(ws), 0 if ws is None else ws.numel(), _stream()), "backward")
         return lv_grad, pos_grad
 
-    def double_backward_from_positions(self, inp, double_positions_grad, grad_sliced_values_monolithic):
+    def double_backward_from_positions(self, inp, double_positions_grad, grad_sliced_values_monolithic,
+                                       want_lattice_values_grad=True):
         """-> (lattice_values_grad (L,C,2), grad_grad_sliced_values (L+E,2,N))
         (reference: Encoding<D,2>::double_backward_from_positions, src/Encoding.cu:219-334).
-        The upstream gradient of the first backward may again be a view of row-major rows."""
+        The upstream gradient of the first backward may again be a view of row-major rows.
+        Without ``want_lattice_values_grad`` only the gathering half runs and the first result is None."""
         fp = self.fixed_params
         pos, lv, shift, win, levels, cap = self._check_common(inp)
         n = pos.shape[0]
@@ -392,8 +458,36 @@ class EncodingWrapper:
         _check_f32_gpu(double_positions_grad, "double_positions_grad", 2)
         _require(double_positions_grad.shape == pos.shape, "double_positions_grad should be nr_positions x pos_dim")
         dpos = double_positions_grad.contiguous()
-        lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device)
         ggs = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
+        if not want_lattice_values_grad:
+            with torch.cuda.device(pos.device):
+                if lv.dtype in TABLE_FORMATS:
+                    _check(lib().penc_double_backward_from_positions_half(
+                        self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), TABLE_FORMATS[lv.dtype],
+                        _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(dpos), _ptr(grad),
+                        0 if grad.is_contiguous() else grad.stride(2), None, _ptr(ggs), int(fp.m_concat_points), None, 0,
+                        _stream()), "double_backward_from_positions")
+                else:
+                    _check(lib().penc_double_backward_from_positions_rowmajor(
+                        self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                        _ptr(win), _ptr(dpos), _ptr(grad), grad.stride(2), None, _ptr(ggs), int(fp.m_concat_points),
+                        None, 0, _stream()) if not grad.is_contiguous() else lib().penc_double_backward_from_positions(
+                        self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                        _ptr(win), _ptr(dpos), _ptr(grad), None, _ptr(ggs), int(fp.m_concat_points), None, 0, _stream()),
+                        "double_backward_from_positions")
+            return None, ggs
+        if self.sparse_table_grad:
+            _require(lv.dtype not in TABLE_FORMATS, "sparse_table_grad needs an fp32 table")
+            sparse = self.sparse_grad_for(lv)
+            with torch.cuda.device(pos.device):
+                ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, nr_feat=self.nr_feat)
+                _check(lib().penc_double_backward_from_positions_sparse(
+                    self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv), _ptr(fp.m_scale_factor), _ptr(shift),
+                    _ptr(win), _ptr(dpos), _ptr(grad), 0 if grad.is_contiguous() else grad.stride(2), _ptr(sparse.grad),
+                    _ptr(sparse.touched), _ptr(ggs), int(fp.m_concat_points), _ptr(ws), 0 if ws is None else ws.numel(),
+                    _stream()), "double_backward_from_positions_sparse")
+            return None, ggs
+        lv_grad = torch.empty(lv.shape, dtype=torch.float32, device=lv.device)
         with torch.cuda.device(pos.device):
             ws = scatter_workspace(self.pos_dim, n, levels, cap, pos.device, nr_feat=self.nr_feat)
             if lv.dtype in TABLE_FORMATS:

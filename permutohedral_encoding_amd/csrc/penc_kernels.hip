@@ -225,7 +225,7 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
     BinTarget bins = bins_of_level(pass_bins, level_in_pass);
     if constexpr (!kWideBins) bins.bin_shift = kBinSlotsLog2;  // a constant from here on
     const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair_level % feat_pairs) * 2,
-                               2 * feat_pairs, bins.records != nullptr ? bins.direct : nullptr, bins.bin_shift};
+                               2 * feat_pairs, bins.direct, bins.bin_shift};
     // Everything a thread reads lies within its group of at most 16 x 512 points, so the addresses are
     // wave-uniform 64-bit bases (scalar registers) plus 32-bit per-thread offsets.
     const uint32_t last_in_group = static_cast<uint32_t>(n_points - 1 - group_base);
@@ -470,6 +470,63 @@ adamw_step_kernel(float* __restrict__ params, const float* __restrict__ grads, f
         params[i] = p;
         exp_avg[i] = m;
         exp_avg_sq[i] = v;
+    }
+}
+
+// The same update, or only the clearing of the gradient, restricted to the slot ranges a caller's map of
+// touched ranges names (the sparse entry points): one workgroup per (slot range, level) looks at the
+// range's flags (one per pair of features) and leaves at once when nothing was added there, so the
+// cost follows what the batch touched and not the size of the table.  Within a touched range an entry
+// with a gradient of exactly 0 is left alone, as with skip_zero.  `clear` zeroes the gradients the
+// workgroup has used and the range's flags, which is what the next accumulation expects.
+template <bool kUpdate, typename Vec>
+__global__ void __launch_bounds__(kBlock)
+touched_ranges_kernel(float* __restrict__ params, float* __restrict__ grads, float* __restrict__ exp_avg,
+                      float* __restrict__ exp_avg_sq, uint32_t capacity, uint32_t nr_feat, uint32_t n_ranges,
+                      uint32_t range_shift, uint32_t* __restrict__ touched, AdamWStep a, int clear) {
+    constexpr uint32_t kPer = sizeof(Vec) / sizeof(float);
+    const uint32_t range = blockIdx.x, level = blockIdx.y, pairs = nr_feat / 2;
+    uint32_t any = 0u;
+    for (uint32_t p = 0; p < pairs; ++p) any |= touched[(static_cast<size_t>(level) * pairs + p) * n_ranges + range];
+    if (any == 0u) return;
+    const uint32_t slot0 = range << range_shift;
+    const uint32_t slots = capacity - slot0 < (1u << range_shift) ? capacity - slot0 : (1u << range_shift);
+    const size_t base = (static_cast<size_t>(level) * capacity + slot0) * nr_feat;  // a multiple of kPer floats (the host checks)
+    const uint32_t n_vec = slots * nr_feat / kPer;
+    Vec* const g_at = reinterpret_cast<Vec*>(grads + base);
+    for (uint32_t i = threadIdx.x; i < n_vec; i += kBlock) {
+        const Vec gv = g_at[i];
+        float g[kPer];
+        __builtin_memcpy(g, &gv, sizeof(gv));
+        bool nonzero = false;
+#pragma unroll
+        for (uint32_t k = 0; k < kPer; ++k) nonzero = nonzero || g[k] != 0.0f;
+        if (!nonzero) continue;
+        if constexpr (kUpdate) {
+            Vec pv = reinterpret_cast<Vec*>(params + base)[i], mv = reinterpret_cast<Vec*>(exp_avg + base)[i],
+                vv = reinterpret_cast<Vec*>(exp_avg_sq + base)[i];
+            float p[kPer], m[kPer], v[kPer];
+            __builtin_memcpy(p, &pv, sizeof(pv));
+            __builtin_memcpy(m, &mv, sizeof(mv));
+            __builtin_memcpy(v, &vv, sizeof(vv));
+#pragma unroll
+            for (uint32_t k = 0; k < kPer; ++k) adamw_update(a, true, g[k], p[k], m[k], v[k]);
+            __builtin_memcpy(&pv, p, sizeof(pv));
+            __builtin_memcpy(&mv, m, sizeof(mv));
+            __builtin_memcpy(&vv, v, sizeof(vv));
+            reinterpret_cast<Vec*>(params + base)[i] = pv;
+            reinterpret_cast<Vec*>(exp_avg + base)[i] = mv;
+            reinterpret_cast<Vec*>(exp_avg_sq + base)[i] = vv;
+        }
+        if (clear) {
+            Vec zero;
+            __builtin_memset(&zero, 0, sizeof(zero));
+            g_at[i] = zero;
+        }
+    }
+    if (clear) {
+        __syncthreads();  // every thread has read the flags
+        if (threadIdx.x < pairs) touched[(static_cast<size_t>(level) * pairs + threadIdx.x) * n_ranges + range] = 0u;
     }
 }
 
@@ -860,11 +917,14 @@ using namespace penc;
 // the [level][feature][n] layout, otherwise the gradient is rows of that many floats.  With
 // double_pos_grad the same for the table-gradient half of the double backward.  grad_level_major (rows
 // only, may be NULL) receives the upstream gradient in [level][feature][n] order as a by-product.
+// With `touched` (the sparse entry points) nothing is cleared: the sums are added to a gradient the caller
+// keeps across calls, and `touched` [pair level][slot range] is that caller's record of the slot ranges
+// that hold anything; it takes the place of the workspace's flags of direct adds.
 static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity, const float* positions,
                           const float* scale_factor, const float* random_shift, const float* anneal_window,
                           const float* grad, int64_t grad_row_stride, const float* double_pos_grad,
                           float* lattice_values_grad, float* grad_level_major, void* workspace, size_t workspace_bytes,
-                          hipStream_t st) {
+                          hipStream_t st, uint32_t* touched = nullptr) {
     const int n = static_cast<int>(nr_positions);
     const uint32_t cap = static_cast<uint32_t>(capacity), mask = mask_of(capacity);
     // every pair of features is scattered like a level of its own (see backward_table_kernel)
@@ -876,9 +936,14 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
         tiles_per_group = kScatterTiles;
         plan = plan_bins(pos_dim, nr_positions, pair_levels, capacity, tiles_per_group, workspace, workspace_bytes);
     }
-    if (int rc = clear_table_grad(lattice_values_grad, pair_levels, capacity, plan.enabled ? plan.target.direct : nullptr,
-                                  plan.direct_bytes, st))
+    if (touched != nullptr) {
+        plan.target.direct = touched;
+        plan.target.n_bins = bins_for_capacity(capacity);
+        plan.target.bin_shift = bin_shift_for_capacity(capacity);
+    } else if (int rc = clear_table_grad(lattice_values_grad, pair_levels, capacity, plan.enabled ? plan.target.direct : nullptr,
+                                         plan.direct_bytes, st)) {
         return rc;
+    }
     uint32_t* const direct_flags = plan.target.direct;
     const int per_pass = plan.enabled ? plan.levels_per_pass : pair_levels;
     const uint32_t dies = dies_of_current_device();
@@ -886,7 +951,7 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
         const int count = pair_levels - first < per_pass ? pair_levels - first : per_pass;
         const unsigned padded_groups = (scatter_groups(nr_positions, tiles_per_group) + dies - 1) / dies * dies;
         const dim3 grid(padded_groups * static_cast<unsigned>(count));
-        if (plan.enabled) plan.target.direct = direct_flags + static_cast<size_t>(first) * plan.target.n_bins;
+        if (direct_flags != nullptr) plan.target.direct = direct_flags + static_cast<size_t>(first) * plan.target.n_bins;
 #define PENC_LAUNCH_TABLE_(ROW_MAJOR, SECOND_ORDER, WIDE)                                                                  \
     PENC_DISPATCH_D(pos_dim, hipLaunchKernelGGL((backward_table_kernel<DD, ROW_MAJOR, SECOND_ORDER, WIDE>), grid,            \
                                                 dim3(kScatterBlock), 0, st, n, first, static_cast<uint32_t>(count),          \
@@ -899,7 +964,7 @@ static int table_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr
     } else {                                             \
         PENC_LAUNCH_TABLE_(ROW_MAJOR, SECOND_ORDER, false); \
     }
-        const bool wide_bins = plan.enabled && plan.target.bin_shift != static_cast<uint32_t>(kBinSlotsLog2);
+        const bool wide_bins = direct_flags != nullptr && plan.target.bin_shift != static_cast<uint32_t>(kBinSlotsLog2);
         if (double_pos_grad != nullptr && grad_row_stride != 0) {
             PENC_LAUNCH_TABLE(true, true);
         } else if (double_pos_grad != nullptr) {
@@ -967,7 +1032,7 @@ static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                          const float* positions, const TableRef& table, const float* scale_factor,
                          const float* random_shift, const float* anneal_window,
                          const float* grad_sliced_values, float* lattice_values_grad, float* positions_grad,
-                         void* workspace, size_t workspace_bytes, void* stream) {
+                         void* workspace, size_t workspace_bytes, void* stream, uint32_t* touched = nullptr) {
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
     if (!positions || !scale_factor || !random_shift || !anneal_window || !grad_sliced_values)
         return PENC_ERR_NULL_POINTER;
@@ -978,7 +1043,7 @@ static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
     if (lattice_values_grad)
         if (int rc = table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
                                     anneal_window, grad_sliced_values, 0, nullptr, lattice_values_grad, nullptr, workspace,
-                                    workspace_bytes, st))
+                                    workspace_bytes, st, touched))
             return rc;
     if (positions_grad)
         return positions_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor,
@@ -1139,7 +1204,7 @@ static int backward_rowmajor_impl(int pos_dim, int nr_feat, int64_t nr_positions
                                   const float* positions, const TableRef& table, const float* scale_factor,
                                   const float* random_shift, const float* anneal_window, const float* grad_rows,
                                   int64_t grad_row_stride, float* lattice_values_grad, float* positions_grad,
-                                  void* workspace, size_t workspace_bytes, void* stream) {
+                                  void* workspace, size_t workspace_bytes, void* stream, uint32_t* touched = nullptr) {
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
     if (!positions || !scale_factor || !random_shift || !anneal_window) return PENC_ERR_NULL_POINTER;
     if (!lattice_values_grad && !positions_grad) return PENC_ERR_NULL_POINTER;
@@ -1150,7 +1215,7 @@ static int backward_rowmajor_impl(int pos_dim, int nr_feat, int64_t nr_positions
     if (!positions_grad)
         return table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
                               anneal_window, grad_rows, grad_row_stride, nullptr, lattice_values_grad, nullptr, workspace,
-                              workspace_bytes, st);
+                              workspace_bytes, st, touched);
     // The position gradient gathers level by level and reads its upstream gradient as [level][feature][n]:
     // that copy lives at the front of the workspace; the rest serves the scatter and then the partial sums.
     const size_t copy_bytes = static_cast<size_t>(nr_levels) * nr_feat * static_cast<size_t>(nr_positions) * sizeof(float);
@@ -1165,7 +1230,7 @@ static int backward_rowmajor_impl(int pos_dim, int nr_feat, int64_t nr_positions
         // the scattering kernel reads every (point, level) pair of the rows anyway and leaves the copy behind
         if (int rc = table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift,
                                     anneal_window, grad_rows, grad_row_stride, nullptr, lattice_values_grad, level_major,
-                                    rest, rest_bytes, st))
+                                    rest, rest_bytes, st, touched))
             return rc;
     } else {
         const int cols = nr_feat * nr_levels;
@@ -1216,7 +1281,7 @@ static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, 
                                 const float* random_shift, const float* anneal_window,
                                 const float* double_positions_grad, const float* grad, int64_t grad_row_stride,
                                 float* lattice_values_grad, float* grad_grad_sliced_values, int concat_points,
-                                void* workspace, size_t workspace_bytes, void* stream) {
+                                void* workspace, size_t workspace_bytes, void* stream, uint32_t* touched = nullptr) {
     const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
     if (!positions || !table.values || !scale_factor || !random_shift || !anneal_window ||
@@ -1238,7 +1303,7 @@ static int double_backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, 
     if (!lattice_values_grad) return PENC_OK;
     return table_backward(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, scale_factor, random_shift, anneal_window,
                           grad, grad_row_stride, double_positions_grad, lattice_values_grad, nullptr, workspace,
-                          workspace_bytes, st);
+                          workspace_bytes, st, touched);
 }
 
 int penc_double_backward_from_positions(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
@@ -1287,12 +1352,8 @@ int penc_double_backward_from_positions_half(int pos_dim, int nr_feat, int64_t n
                                 concat_points, workspace, workspace_bytes, stream);
 }
 
-int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* exp_avg_sq, int64_t n, double lr,
-                    double beta1, double beta2, double eps, double weight_decay, int64_t step, int skip_zero_gradients,
-                    void* stream) {
-    if (!params || !grads || !exp_avg || !exp_avg_sq) return PENC_ERR_NULL_POINTER;
-    if (n <= 0 || step <= 0) return PENC_ERR_BAD_SIZE;
-    // the scalars as torch.optim.AdamW forms them (in double), rounded once for the kernel
+// The scalars of one AdamW step as torch.optim.AdamW forms them (in double), rounded once for the kernel.
+static AdamWStep adamw_scalars(double lr, double beta1, double beta2, double eps, double weight_decay, int64_t step) {
     AdamWStep a;
     a.decay = static_cast<float>(1.0 - lr * weight_decay);
     a.one_minus_b1 = static_cast<float>(1.0 - beta1);
@@ -1301,6 +1362,15 @@ int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* ex
     a.step_size = static_cast<float>(lr / (1.0 - __builtin_pow(beta1, static_cast<double>(step))));
     a.inv_c2 = static_cast<float>(1.0 / __builtin_sqrt(1.0 - __builtin_pow(beta2, static_cast<double>(step))));
     a.eps = static_cast<float>(eps);
+    return a;
+}
+
+int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* exp_avg_sq, int64_t n, double lr,
+                    double beta1, double beta2, double eps, double weight_decay, int64_t step, int skip_zero_gradients,
+                    void* stream) {
+    if (!params || !grads || !exp_avg || !exp_avg_sq) return PENC_ERR_NULL_POINTER;
+    if (n <= 0 || step <= 0) return PENC_ERR_BAD_SIZE;
+    const AdamWStep a = adamw_scalars(lr, beta1, beta2, eps, weight_decay, step);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const uintptr_t all = reinterpret_cast<uintptr_t>(params) | reinterpret_cast<uintptr_t>(grads) |
                           reinterpret_cast<uintptr_t>(exp_avg) | reinterpret_cast<uintptr_t>(exp_avg_sq);
@@ -1323,6 +1393,84 @@ int penc_adamw_step(float* params, const float* grads, float* exp_avg, float* ex
         if (int rc = check_launch()) return rc;
     }
     return PENC_OK;
+}
+
+size_t penc_touched_map_entries(int nr_feat, int nr_levels, int capacity) {
+    if ((nr_feat != 2 && nr_feat != 4 && nr_feat != 8) || nr_levels <= 0 || capacity <= 0) return 0;
+    return static_cast<size_t>(nr_levels) * (nr_feat / 2) * bins_for_capacity(capacity);
+}
+
+int penc_touched_range_slots(int capacity) { return capacity > 0 ? 1 << bin_shift_for_capacity(capacity) : 0; }
+
+int penc_backward_sparse(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                         const float* positions, const float* lattice_values, const float* scale_factor,
+                         const float* random_shift, const float* anneal_window, const float* grad, int64_t grad_row_stride,
+                         float* lattice_values_grad, uint32_t* touched, float* positions_grad, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+    if (!lattice_values_grad || !touched) return PENC_ERR_NULL_POINTER;
+    const TableRef table{lattice_values, 0};
+    if (grad_row_stride != 0)
+        return backward_rowmajor_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor,
+                                      random_shift, anneal_window, grad, grad_row_stride, lattice_values_grad, positions_grad,
+                                      workspace, workspace_bytes, stream, touched);
+    return backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, table, scale_factor, random_shift,
+                         anneal_window, grad, lattice_values_grad, positions_grad, workspace, workspace_bytes, stream, touched);
+}
+
+int penc_double_backward_from_positions_sparse(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                                               const float* positions, const float* lattice_values,
+                                               const float* scale_factor, const float* random_shift,
+                                               const float* anneal_window, const float* double_positions_grad,
+                                               const float* grad, int64_t grad_row_stride, float* lattice_values_grad,
+                                               uint32_t* touched, float* grad_grad_sliced_values, int concat_points,
+                                               void* workspace, size_t workspace_bytes, void* stream) {
+    if (!lattice_values_grad || !touched) return PENC_ERR_NULL_POINTER;
+    if (grad_row_stride != 0 && nr_levels > 0 && nr_positions > 0)
+        if (int rc = check_rows(grad, grad_row_stride, nr_positions, nr_levels, nr_feat)) return rc;
+    return double_backward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
+                                scale_factor, random_shift, anneal_window, double_positions_grad, grad, grad_row_stride,
+                                lattice_values_grad, grad_grad_sliced_values, concat_points, workspace, workspace_bytes, stream,
+                                touched);
+}
+
+// The launch shared by penc_adamw_step_sparse and penc_clear_touched: one workgroup per (slot range, level).
+static int launch_touched_ranges(bool update, float* params, float* grads, float* exp_avg, float* exp_avg_sq, int nr_feat,
+                                 int nr_levels, int capacity, uint32_t* touched, const AdamWStep& a, int clear, void* stream) {
+    if (!grads || !touched || (update && (!params || !exp_avg || !exp_avg_sq))) return PENC_ERR_NULL_POINTER;
+    if ((nr_feat != 2 && nr_feat != 4 && nr_feat != 8)) return PENC_ERR_UNSUPPORTED_NR_FEAT;
+    if (nr_levels <= 0 || nr_levels > 65535 || capacity <= 0) return PENC_ERR_BAD_SIZE;
+    const uintptr_t all = reinterpret_cast<uintptr_t>(grads) |
+                          (update ? reinterpret_cast<uintptr_t>(params) | reinterpret_cast<uintptr_t>(exp_avg) |
+                                        reinterpret_cast<uintptr_t>(exp_avg_sq)
+                                  : uintptr_t{0});
+    if ((all & 7u) != 0) return PENC_ERR_MISALIGNED;
+    const uint32_t n_ranges = bins_for_capacity(capacity), shift = bin_shift_for_capacity(capacity);
+    // 16 bytes at a time where every level's first value is 16-byte aligned, else 8 (a slot of two features)
+    const bool wide = (all & 15u) == 0 && (static_cast<int64_t>(capacity) * nr_feat) % 4 == 0;
+    const dim3 grid(n_ranges, static_cast<unsigned>(nr_levels));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PENC_LAUNCH_TOUCHED(UPDATE, VEC)                                                                                   \
+    hipLaunchKernelGGL((touched_ranges_kernel<UPDATE, VEC>), grid, dim3(kBlock), 0, st, params, grads, exp_avg, exp_avg_sq, \
+                       static_cast<uint32_t>(capacity), static_cast<uint32_t>(nr_feat), n_ranges, shift, touched, a, clear)
+    if (update && wide) PENC_LAUNCH_TOUCHED(true, float4);
+    else if (update) PENC_LAUNCH_TOUCHED(true, float2);
+    else if (wide) PENC_LAUNCH_TOUCHED(false, float4);
+    else PENC_LAUNCH_TOUCHED(false, float2);
+#undef PENC_LAUNCH_TOUCHED
+    return check_launch();
+}
+
+int penc_adamw_step_sparse(float* params, float* grads, float* exp_avg, float* exp_avg_sq, int nr_feat, int nr_levels,
+                           int capacity, uint32_t* touched, double lr, double beta1, double beta2, double eps,
+                           double weight_decay, int64_t step, int clear, void* stream) {
+    if (step <= 0) return PENC_ERR_BAD_SIZE;
+    return launch_touched_ranges(true, params, grads, exp_avg, exp_avg_sq, nr_feat, nr_levels, capacity, touched,
+                                 adamw_scalars(lr, beta1, beta2, eps, weight_decay, step), clear, stream);
+}
+
+int penc_clear_touched(float* grads, int nr_feat, int nr_levels, int capacity, uint32_t* touched, void* stream) {
+    return launch_touched_ranges(false, nullptr, grads, nullptr, nullptr, nr_feat, nr_levels, capacity, touched, AdamWStep{}, 1,
+                                 stream);
 }
 
 int penc_transpose(const float* src, float* dst, int64_t rows, int cols, void* stream) {

@@ -98,9 +98,12 @@ constexpr size_t kSplitRecordBytes = sizeof(RecordValues) + sizeof(uint16_t);
 //   records [level_in_pass][bin][group][segment_capacity]   12-byte records, or the 8-byte values of split ones
 //   slots   [level_in_pass][bin][group][segment_capacity]   the 2-byte slots of split records; nullptr otherwise
 //   counts  [level_in_pass][bin][group]            records actually written (<= segment_capacity)
-//   direct  [level_in_pass][bin]                   nonzero once anything has been added straight into the gradient
-//                                                  in the bin's slot range (cleared with the gradient; see GradSlice)
-// `records` == nullptr disables binning.
+//   direct  [level_in_pass][bin]                   nonzero once anything has been added into the gradient in the
+//                                                  bin's slot range: straight from the scattering kernel (see
+//                                                  GradSlice), or by the bin's reducer.  Cleared with the gradient, or,
+//                                                  for a caller who keeps gradient and flags across calls (the sparse
+//                                                  entry points), the caller's map of touched slot ranges.
+// `records` == nullptr disables binning (`direct`, `n_bins` and `bin_shift` may still be set: flags without bins).
 struct BinTarget {
     void* records;
     uint16_t* slots;
@@ -121,8 +124,8 @@ __device__ __forceinline__ BinTarget bins_of_level(const BinTarget& pass, uint32
         t.records = static_cast<char*>(pass.records) + records * (pass.slots != nullptr ? sizeof(RecordValues) : sizeof(BinRecord));
         if (pass.slots != nullptr) t.slots += records;
         t.counts += segments;
-        t.direct += static_cast<size_t>(k) * pass.n_bins;
     }
+    if (pass.direct != nullptr) t.direct += static_cast<size_t>(k) * pass.n_bins;
     return t;
 }
 
@@ -1108,13 +1111,15 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
             add(b, got_b);
         }
     }
+    // nothing has been added to the bin's slots since the gradient was cleared (or, for a caller who keeps the gradient
+    // across calls, since that caller last cleared this slot range): the sums are the result.  Read before the barrier:
+    // thread 0 sets the flag at the end.
+    const bool untouched_so_far = bins.direct[bin] == 0u;
     __syncthreads();
     const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr, 0u};
     const uint32_t slot0 = bin << kBinSlotsLog2;  // (this kernel serves bins of kBinSlots slots only)
     const bool alone = gridDim.z == 1;
     if (alone) {
-        // nothing but this workgroup has added to the bin's slots since the gradient was cleared: the sums are the result
-        const bool untouched_so_far = bins.direct[bin] == 0u;
         // all of a thread's read-modify-writes at once: the loads are issued together, not one per trip
         constexpr int kMine = kBinSlots / kReduceBlock;
         float2 sum[kMine], g[kMine];
@@ -1141,8 +1146,10 @@ bin_reduce_kernel(BinTarget pass_bins, const float* __restrict__ window, uint32_
                 *reinterpret_cast<float2*>(level_grad.at(slot0 + s)) = g[k];
             }
         }
+        if (threadIdx.x == 0 && untouched_so_far) bins.direct[bin] = 1u;  // this slot range now holds sums
         return;
     }
+    if (threadIdx.x == 0 && untouched_so_far) bins.direct[bin] = 1u;  // (the workgroups that share the bin all store the same value)
     for (uint32_t s = threadIdx.x; s < static_cast<uint32_t>(kBinSlots); s += kReduceBlock) {
         const double v0 = acc0[s], v1 = acc1[s];
         if ((v0 != 0.0 || v1 != 0.0) && slot0 + s < capacity) {
@@ -1286,6 +1293,7 @@ bin_reduce_levels_kernel(BinTarget pass_bins, const float* __restrict__ window, 
         const GradSlice level_grad{table_grad + (static_cast<size_t>(level) * capacity * feat_pairs + pair) * 2, 2 * feat_pairs, nullptr, 0u};
         const uint32_t slot0 = (bin << pass_bins.bin_shift) + (range << kBinSlotsLog2);
         const bool untouched_so_far = ((direct_mask >> i) & 1u) == 0u;
+        if (threadIdx.x == 0 && untouched_so_far) pass_bins.direct[static_cast<size_t>(level_in_pass(i)) * n_bins + bin] = 1u;  // this slot range now holds sums
         constexpr int kMine = kBinSlots / kReduceBlock;
         // (two loops, so that the usual one has no load to wait for: a wait would also be one for the
         // records of the next step, which are on their way)

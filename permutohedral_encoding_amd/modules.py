@@ -21,12 +21,21 @@ class PermutoEncoding(torch.nn.Module):
     refreshed whenever the parameter has been modified in place (optimizer steps), so it pays for
     large tables and for inference.  float16 resolves the reference's initial values (about 1e-5)
     only to 6e-8; bfloat16 keeps three significant digits at any magnitude.
+
+    ``sparse_table_grad=True`` is for tables that dwarf the batch: the gradient w.r.t. ``lattice_values``
+    is not handed to autograd (``lattice_values.grad`` stays None) but added into ``table_grad``, a
+    gradient array the module keeps across steps together with a map of the slot ranges that hold
+    anything; ``permutohedral_encoding_amd.optim.SparseTableAdamW`` steps the table from it and zeroes
+    what was touched.  Neither the gradient calls nor the optimizer then walk the whole table (the
+    reference clears a dense gradient in every call, src/Encoding.cu:141, 246, and its training
+    protocol steps the whole table, examples/performance.py:99-101).
     """
 
     def __init__(self, pos_dim, capacity, nr_levels, nr_feat_per_level, scale_per_level,
                  appply_random_shift_per_level=True, concat_points=False, concat_points_scaling=1.0, device=None,
-                 lattice_half_precision=False):
+                 lattice_half_precision=False, sparse_table_grad=False):
         super().__init__()
+        self.sparse_table_grad = bool(sparse_table_grad)
         if lattice_half_precision in (None, False):
             self.lattice_half_precision = None
         elif lattice_half_precision is True or lattice_half_precision == torch.float16:
@@ -74,7 +83,13 @@ class PermutoEncoding(torch.nn.Module):
                                                    self.concat_points, self.concat_points_scaling)
         lattice = _native.EncodingWrapper.create(self.pos_dim, self.nr_feat_per_level, fixed_params)
         lattice.half_table = getattr(self, "lattice_half_precision", None)
+        lattice.sparse_table_grad = getattr(self, "sparse_table_grad", False)
         return fixed_params, lattice
+
+    @property
+    def table_grad(self):
+        """With ``sparse_table_grad``: the ``SparseTableGrad`` the gradient calls add into (None before the first one)."""
+        return self.lattice.sparse_grad
 
     def __getstate__(self):
         state = self.__dict__.copy()

@@ -475,3 +475,89 @@ def test_training_with_the_fused_optimizer_and_a_half_precision_table():
         losses.append(loss.item())
     assert losses[-1] < 0.9 * losses[0], losses
     assert all(later < earlier for earlier, later in zip(losses, losses[1:])), losses
+
+
+def test_sparse_table_grad_module_and_optimizer_follow_the_dense_path():
+    """PermutoEncoding(sparse_table_grad=True) with SparseTableAdamW against the same module with dense
+    gradients: an eikonal-style step (backward and double backward both reach the table) leaves
+    lattice_values.grad None and the sum of the two gradients in table_grad; the sparse step equals
+    torch.optim.AdamW on every slot that received a gradient and leaves every other slot, its moments
+    included, alone; gradient and map are zero again afterwards."""
+    import permutohedral_encoding_amd as pe
+    from permutohedral_encoding_amd.optim import SparseTableAdamW
+    cap, levels, n = 1 << 16, 5, 3000
+    sig = np.geomspace(1.0, 5e-3, levels)
+    torch.manual_seed(1)
+    dense = pe.PermutoEncoding(3, cap, levels, 2, sig)
+    sparse = pe.PermutoEncoding(3, cap, levels, 2, sig, sparse_table_grad=True)
+    with torch.no_grad():
+        dense.lattice_values.uniform_(-1, 1)
+        sparse.lattice_values.copy_(dense.lattice_values)
+        sparse.random_shift_per_level.copy_(dense.random_shift_per_level)
+    start = dense.lattice_values.detach().clone()
+    kw = dict(lr=1e-2, betas=(0.9, 0.99), eps=1e-12, weight_decay=0.01)
+    opt_dense, opt_sparse = torch.optim.AdamW([dense.lattice_values], **kw), SparseTableAdamW(sparse, **kw)
+    pts = torch.rand(n, 3, device="cuda")
+    a = torch.randn(dense.output_dims(), device="cuda")
+
+    def loss_of(m):
+        pos = pts.clone().requires_grad_(True)
+        sdf = (m(pos) * a).sum(dim=1)
+        grad_pos, = torch.autograd.grad(sdf.sum(), pos, create_graph=True)
+        return ((grad_pos.norm(dim=1) - 1.0) ** 2).mean() + 1e-3 * (sdf ** 2).mean()
+
+    for step in range(3):  # the same points every step: the same slots are touched, so the two optimizers agree on them
+        opt_dense.zero_grad()
+        loss_of(dense).backward()
+        loss_of(sparse).backward()
+        assert sparse.lattice_values.grad is None
+        g_dense, g_sparse = dense.lattice_values.grad, sparse.table_grad.grad
+        scale = g_dense.abs().max().item()
+        assert torch.allclose(g_sparse, g_dense, rtol=1e-4, atol=1e-5 * scale), (step, (g_sparse - g_dense).abs().max().item())
+        touched = g_dense != 0
+        assert torch.equal(g_sparse != 0, touched) or (g_sparse != 0)[~touched].sum() == 0
+        opt_dense.step()
+        opt_sparse.step()
+        assert not sparse.table_grad.grad.any().item() and not sparse.table_grad.touched.any().item()
+        got, want = sparse.lattice_values.detach(), dense.lattice_values.detach()
+        assert torch.allclose(got[touched], want[touched], rtol=1e-4, atol=1e-6), (step, (got - want)[touched].abs().max().item())
+        assert torch.equal(got[~touched], start[~touched])
+    state = opt_sparse.state[sparse.lattice_values]
+    assert state["step"] == 3 and torch.all(state["exp_avg"][~touched] == 0) and torch.all(state["exp_avg_sq"][~touched] == 0)
+    with pytest.raises(ValueError):
+        SparseTableAdamW(dense)
+
+
+def test_gradients_no_pass_consumes_are_not_computed():
+    """autograd.grad(sdf, positions, create_graph=True) runs the first-order backward of the slicing, but
+    nothing in that pass uses the table gradient: the library is then asked for the position gradient
+    alone (the reference launches its table scatter regardless, src/Encoding.cu:167).  The later
+    loss.backward() does ask for it, and a frozen table is never given a second-order gradient."""
+    m = make_module(levels=4)
+    calls, doubles = [], []
+    backward, double = m.lattice.backward, m.lattice.double_backward_from_positions
+
+    def spy_backward(inp, grad):
+        calls.append((inp.m_require_lattice_values_grad, inp.m_require_positions_grad))
+        return backward(inp, grad)
+
+    def spy_double(inp, dpos, grad, want_lattice_values_grad=True):
+        doubles.append(want_lattice_values_grad)
+        return double(inp, dpos, grad, want_lattice_values_grad=want_lattice_values_grad)
+
+    m.lattice.backward, m.lattice.double_backward_from_positions = spy_backward, spy_double
+    pos = torch.rand(800, 3, device="cuda", requires_grad=True)
+    a = torch.randn(m.output_dims(), device="cuda")
+    sdf = (m(pos) * a).sum(dim=1)
+    grad_pos, = torch.autograd.grad(sdf.sum(), pos, create_graph=True)
+    assert calls == [(False, True)]
+    (((grad_pos.norm(dim=1) - 1.0) ** 2).sum() + (sdf ** 2).sum()).backward()
+    assert calls == [(False, True), (True, True)] and doubles == [True]
+    assert m.lattice_values.grad is not None and pos.grad is not None
+    # a frozen table: the double backward runs its gathering half only
+    m.lattice_values.requires_grad_(False)
+    calls.clear(), doubles.clear()
+    sdf = (m(pos) * a).sum(dim=1)
+    grad_pos, = torch.autograd.grad(sdf.sum(), pos, create_graph=True)
+    ((grad_pos.norm(dim=1) - 1.0) ** 2).sum().backward()
+    assert calls == [(False, True)] and doubles == [False]

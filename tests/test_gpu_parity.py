@@ -930,3 +930,66 @@ def test_random_geometry_all_phases_match_oracle(seed, monkeypatch):
     wd = orc.double_backward(p["pos"], p["table"], sf, p["shift"], p["window"], p["dpos"], p["grad"], want_abs=True)
     assert_sum_close(tg2.cpu().numpy(), wd["grad64"], wd["abs64"], SUM_RTOL, f"second-order table gradient, {what}")
     check_grad_grad(ggs.cpu().numpy(), wd)
+
+
+# ----------------------------------------------------------------------------- sparse table gradient
+
+def _touched_slots(sparse, level, pair):
+    """Boolean (capacity,) array: slots whose range the map marks, for one level and pair of features."""
+    m = sparse.touched_map()[level, pair].cpu().numpy() != 0
+    return np.repeat(m, sparse.range_slots)[:sparse.capacity]
+
+
+@pytest.mark.parametrize("d,feat,cap,n,levels,rows", [
+    (3, 2, 1 << 18, 150000, 5, False),     # binned, slot ranges of 8192
+    (4, 4, 100003, 60000, 3, True),        # not a power of two, two pairs of features, row-major upstream gradient
+    (3, 2, 1 << 23, 120000, 3, False),     # ranges wider than a reducer's LDS
+    (5, 2, 1 << 20, 3000, 4, False),       # too few contributions for binning: every add goes straight into the gradient
+    (2, 8, 5000, 20000, 6, True),          # a single slot range per level
+])
+def test_sparse_table_gradient_accumulates_and_is_cleared(d, feat, cap, n, levels, rows):
+    """penc_backward_sparse and penc_double_backward_from_positions_sparse add into one gradient kept
+    across calls and mark the slot ranges they reach; penc_clear_touched restores the all-zero state.
+    Twice in a row, the second time with fewer points, against the oracle's sums."""
+    from permutohedral_encoding_amd import _native
+    p = random_problem(d, n, levels, 1, seed=77 + d, sigma_range=(1.0, 2e-3), nr_feat=feat)
+    if levels > 3:
+        p["window"][2] = 0.0  # a masked level touches nothing
+    p["table"] = np.random.default_rng(3).uniform(-1, 1, (levels, cap, feat)).astype(np.float32)
+    sf = orc.scale_factors(d, p["sigmas"])
+    enc, _ = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
+    enc.sparse_table_grad = True
+    table = to_gpu(p["table"])
+    for count in (n, n // 3):
+        pos, dpos = p["pos"][:count], p["dpos"][:count]
+        grad = np.ascontiguousarray(p["grad"][:, :, :count])
+        inp = _native.EncodingInput(table, to_gpu(pos), to_gpu(p["window"]), True, True)
+        g_dev = to_gpu(grad)
+        if rows:  # the (L, F, N) view of rows (N, F*L) autograd hands over
+            g_dev = to_gpu(np.ascontiguousarray(grad.transpose(2, 0, 1).reshape(count, -1))).view(count, levels, feat).permute(1, 2, 0)
+        tg, pg = enc.backward(inp, g_dev)
+        assert tg is None
+        sparse = enc.sparse_grad
+        first = orc.backward_table(pos, sf, p["shift"], p["window"], grad, cap, want_abs=True)
+        assert_sum_close(sparse.grad.cpu().numpy(), first["grad64"], first["abs64"], SUM_RTOL, "sparse table gradient")
+        check_pos_grad(pg.cpu().numpy(), orc.backward_pos(pos, p["table"], sf, p["shift"], p["window"], grad))
+        tg2, ggs = enc.double_backward_from_positions(inp, to_gpu(dpos), g_dev)
+        assert tg2 is None and enc.sparse_grad is sparse
+        second = orc.double_backward(pos, p["table"], sf, p["shift"], p["window"], dpos, grad, want_abs=True)
+        check_grad_grad(ggs.cpu().numpy(), second)
+        got = sparse.grad.cpu().numpy()
+        assert_sum_close(got, first["grad64"] + second["grad64"], first["abs64"] + second["abs64"], SUM_RTOL,
+                         "sum of the two sparse table gradients")
+        # the map covers every slot that holds anything, and a masked level is not marked at all
+        for level in range(levels):
+            for pair in range(feat // 2):
+                marked = _touched_slots(sparse, level, pair)
+                held = np.any(got[level][:, 2 * pair:2 * pair + 2] != 0, axis=1)
+                assert not np.any(held & ~marked), (level, pair)
+                if p["window"][level] == 0.0:
+                    assert not marked.any()
+        sparse.clear()
+        assert not sparse.touched.any().item() and not sparse.grad.any().item()
+    enc.sparse_table_grad = False
+    tg, _ = enc.backward(_native.EncodingInput(table, to_gpu(p["pos"]), to_gpu(p["window"]), True, False), to_gpu(p["grad"]))
+    assert tg is not None  # the dense path is untouched by the switch
