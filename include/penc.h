@@ -55,7 +55,7 @@ extern "C" {
 #define PENC_ERR_MISALIGNED 5          /* lattice_values not aligned to a slot, or a gradient array not to 8 bytes */
 #define PENC_ERR_LAUNCH 6              /* the HIP runtime rejected a launch (hipGetLastError) */
 #define PENC_ERR_SCRATCH_TOO_SMALL 7    /* penc_backward_static: the problem does not fit the static scratch */
-#define PENC_ERR_WORKSPACE_TOO_SMALL 8  /* penc_backward_rowmajor with positions_grad: no room for the level-major copy */
+#define PENC_ERR_WORKSPACE_TOO_SMALL 8  /* penc_backward_rowmajor with positions_grad, penc_forward_rowmajor: no room for the level-major array */
 #define PENC_ERR_UNSUPPORTED_TABLE_FORMAT 9 /* the *_half entry points: table_format is neither PENC_TABLE_FP16 nor PENC_TABLE_BF16 */
 
 const char* penc_status_string(int status);
@@ -101,6 +101,21 @@ int penc_forward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, 
                  const float* positions, const float* lattice_values, const float* scale_factor,
                  const float* random_shift, const float* anneal_window, float* sliced_values,
                  int concat_points, float points_scaling, void* stream);
+
+/* penc_forward with the result as the layer after the encoding reads it: rows
+ * sliced_rows[n][nr_feat*level + feature] of row_stride floats (>= nr_feat*(L+E)) instead of [L+E][F][N].
+ * The gathering kernel keeps working a level at a time (one level's slice of the table stays in L2, its
+ * stores are coalesced) into `workspace`, which must hold the [L+E][F][N] array
+ * (penc_forward_rowmajor_workspace_bytes; PENC_ERR_WORKSPACE_TOO_SMALL otherwise), and an LDS-tiled
+ * transpose then writes every row as one contiguous chunk, at streaming speed.
+ * Replaces: Encoding<D,2>::forward (src/Encoding.cu:55-108) followed by the strided copy a consumer of
+ * contiguous rows makes of the reference's permute + reshape (src/pytorch_modules/modules.py:87); a
+ * consumer that takes the strided view as it is (a matrix multiplication) needs neither. */
+size_t penc_forward_rowmajor_workspace_bytes(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int concat_points);
+int penc_forward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                          const float* positions, const float* lattice_values, const float* scale_factor,
+                          const float* random_shift, const float* anneal_window, float* sliced_rows, int64_t row_stride,
+                          int concat_points, float points_scaling, void* workspace, size_t workspace_bytes, void* stream);
 
 /* First backward.  lattice_values_grad and positions_grad are each optional (NULL = not wanted,
  * the reference's require_*_grad flags); at least one must be given.  lattice_values_grad is

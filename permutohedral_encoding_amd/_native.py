@@ -26,6 +26,10 @@ _SIGNATURES = {
     "penc_forward": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                     _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p,
                                     ctypes.c_int, ctypes.c_float, ctypes.c_void_p]),
+    "penc_forward_rowmajor_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int]),
+    "penc_forward_rowmajor": (ctypes.c_int, [ctypes.c_int, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                             _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, _c_f32p, ctypes.c_int64,
+                                             ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]),
     "penc_scatter_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                                        ctypes.c_int]),
     "penc_positions_workspace_bytes": (ctypes.c_size_t, [ctypes.c_int, ctypes.c_int64, ctypes.c_int]),
@@ -313,6 +317,8 @@ class EncodingWrapper:
     # wrapper keeps across calls, and the gradient calls return None for them
     sparse_table_grad = False
     sparse_grad = None
+    # set by the module (contiguous_output=True): the forward writes rows (N, F(L+E)) and returns a (L+E, F, N) view of them
+    rows_output = False
 
     def sparse_grad_for(self, lattice_values):
         if self.sparse_grad is None or not self.sparse_grad.matches(lattice_values):
@@ -375,6 +381,19 @@ class EncodingWrapper:
         pos, lv, shift, win, levels, cap = self._check_common(inp)
         n = pos.shape[0]
         extra = extra_levels(self.pos_dim, self.nr_feat, fp.m_concat_points)
+        if self.rows_output and lv.dtype not in TABLE_FORMATS and self.nr_feat * (levels + extra) <= 255:
+            # rows[n][F*level + feature], handed back as the (L+E, F, N) view of them: the module's
+            # permute + reshape of that view is the contiguous (N, F(L+E)) array itself
+            cols = self.nr_feat * (levels + extra)
+            rows = torch.empty((n, cols), dtype=torch.float32, device=pos.device)
+            with torch.cuda.device(pos.device):
+                nbytes = int(lib().penc_forward_rowmajor_workspace_bytes(self.pos_dim, self.nr_feat, n, levels, int(fp.m_concat_points)))
+                ws = torch.empty(nbytes, dtype=torch.uint8, device=pos.device)
+                _check(lib().penc_forward_rowmajor(self.pos_dim, self.nr_feat, n, levels, cap, _ptr(pos), _ptr(lv),
+                                                   _ptr(fp.m_scale_factor), _ptr(shift), _ptr(win), _ptr(rows), cols,
+                                                   int(fp.m_concat_points), fp.m_points_scaling, _ptr(ws), nbytes, _stream()),
+                       "forward_rowmajor")
+            return rows.view(n, levels + extra, self.nr_feat).permute(1, 2, 0)
         out = torch.empty((levels + extra, self.nr_feat, n), dtype=torch.float32, device=pos.device)
         with torch.cuda.device(pos.device):
             if lv.dtype in TABLE_FORMATS:

@@ -599,6 +599,36 @@ transpose_kernel(const float* __restrict__ src, int64_t src_row_stride, float* _
         for (int col = wave; col < cols; col += kBlock / 64) dst[static_cast<int64_t>(col) * rows + row0 + lane] = tile[lane * stride + col];
 }
 
+// The other direction: dst[r][c] = src[c][r], from the [level][feature][n] layout the forward writes to rows
+// dst[n][F * level + feature] of `dst_row_stride` floats (what a layer that wants contiguous rows reads; the
+// reference's permute + reshape, src/pytorch_modules/modules.py:87, leaves that copy to the consumer).  Every
+// read is a run of 64 consecutive floats, the write one contiguous chunk when the rows are dense.
+__global__ void __launch_bounds__(kBlock)
+transpose_to_rows_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t dst_row_stride, int64_t rows, int cols) {
+    extern __shared__ float tile[];  // kTransposeRows x (cols | 1)
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * kTransposeRows;
+    const int n_rows = rows - row0 < kTransposeRows ? static_cast<int>(rows - row0) : kTransposeRows;
+    const int stride = cols | 1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane < n_rows)
+        for (int col = wave; col < cols; col += kBlock / 64)
+            tile[lane * stride + col] = __builtin_nontemporal_load(src + static_cast<int64_t>(col) * rows + row0 + lane);
+    __syncthreads();
+    float* chunk = dst + row0 * dst_row_stride;
+    const int n_values = n_rows * cols;
+    int r = threadIdx.x / cols, c = threadIdx.x % cols;
+    const int dr = kBlock / cols, dc = kBlock % cols;
+    for (int i = threadIdx.x; i < n_values; i += kBlock) {
+        chunk[r * dst_row_stride + c] = tile[r * stride + c];
+        r += dr;
+        c += dc;
+        if (c >= cols) {
+            c -= cols;
+            ++r;
+        }
+    }
+}
+
 // Clears two arrays (the second may be empty): n2 and m2 count 8-byte units.
 __global__ void __launch_bounds__(kBlock) fill_zero_kernel(float2* __restrict__ p, size_t n2, float2* __restrict__ q, size_t m2) {
     const size_t stride = static_cast<size_t>(gridDim.x) * kBlock, first = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x;
@@ -1026,6 +1056,14 @@ static int transpose_rows(const float* src, int64_t src_row_stride, float* dst, 
     return check_launch();
 }
 
+static int transpose_to_rows(const float* src, float* dst, int64_t dst_row_stride, int64_t rows, int cols, hipStream_t st) {
+    const size_t lds = static_cast<size_t>(kTransposeRows) * (cols | 1) * sizeof(float);
+    if (cols <= 0 || cols > 255 || lds > 64 * 1024) return PENC_ERR_BAD_SIZE;
+    const unsigned blocks = static_cast<unsigned>((rows + kTransposeRows - 1) / kTransposeRows);
+    hipLaunchKernelGGL(transpose_to_rows_kernel, dim3(blocks), dim3(kBlock), lds, st, src, dst, dst_row_stride, rows, cols);
+    return check_launch();
+}
+
 // penc_backward and penc_backward_static: argument checks, then the table gradient (clear, scatter,
 // reduce) and the position gradient on the same stream.
 static int backward_impl(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
@@ -1082,7 +1120,7 @@ const char* penc_status_string(int status) {
         case PENC_ERR_UNSUPPORTED_NR_FEAT: return "nr_feat_per_level must be 2, 4 or 8";
         case PENC_ERR_MISALIGNED: return "lattice_values must be aligned to one slot (at most 16 bytes), lattice_values_grad and gradient rows to 8 bytes";
         case PENC_ERR_LAUNCH: return "the HIP runtime rejected a kernel launch";
-        case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major copy of the upstream gradient (penc_backward_rowmajor_workspace_bytes)";
+        case PENC_ERR_WORKSPACE_TOO_SMALL: return "the workspace cannot hold the level-major array the call needs (penc_backward_rowmajor_workspace_bytes, penc_forward_rowmajor_workspace_bytes)";
         case PENC_ERR_UNSUPPORTED_TABLE_FORMAT: return "table_format must be PENC_TABLE_FP16 or PENC_TABLE_BF16";
         case PENC_ERR_SCRATCH_TOO_SMALL: return "the problem is too large for the library's static scratch (penc_static_scratch_bytes): use penc_backward with a workspace";
         default: return "unknown status";
@@ -1137,6 +1175,31 @@ int penc_forward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, 
                  int concat_points, float points_scaling, void* stream) {
     return forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0},
                         scale_factor, random_shift, anneal_window, sliced_values, concat_points, points_scaling, stream);
+}
+
+size_t penc_forward_rowmajor_workspace_bytes(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int concat_points) {
+    if (pos_dim < 2 || pos_dim > 8 || (nr_feat != 2 && nr_feat != 4 && nr_feat != 8) || nr_positions <= 0 || nr_levels <= 0) return 0;
+    const size_t cols = static_cast<size_t>(nr_feat) * (nr_levels + penc_extra_levels(pos_dim, nr_feat, concat_points));
+    return cols * static_cast<size_t>(nr_positions) * sizeof(float) + 256;
+}
+
+int penc_forward_rowmajor(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,
+                          const float* positions, const float* lattice_values, const float* scale_factor,
+                          const float* random_shift, const float* anneal_window, float* sliced_rows, int64_t row_stride,
+                          int concat_points, float points_scaling, void* workspace, size_t workspace_bytes, void* stream) {
+    const int extra = penc_extra_levels(pos_dim, nr_feat, concat_points);
+    if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, extra)) return rc;
+    if (!sliced_rows) return PENC_ERR_NULL_POINTER;
+    const int cols = nr_feat * (nr_levels + extra);
+    if (cols > 255 || row_stride < cols || row_stride * nr_positions >= (int64_t{1} << 31)) return PENC_ERR_BAD_SIZE;
+    const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + 255u) & ~uintptr_t{255};
+    const size_t need = static_cast<size_t>(cols) * static_cast<size_t>(nr_positions) * sizeof(float);
+    if (workspace == nullptr || workspace_bytes < (base - reinterpret_cast<uintptr_t>(workspace)) + need) return PENC_ERR_WORKSPACE_TOO_SMALL;
+    float* level_major = reinterpret_cast<float*>(base);
+    if (int rc = forward_impl(pos_dim, nr_feat, nr_positions, nr_levels, capacity, positions, TableRef{lattice_values, 0}, scale_factor,
+                              random_shift, anneal_window, level_major, concat_points, points_scaling, stream))
+        return rc;
+    return transpose_to_rows(level_major, sliced_rows, row_stride, nr_positions, cols, static_cast<hipStream_t>(stream));
 }
 
 int penc_forward_half(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels, int capacity,

@@ -22,6 +22,10 @@ class PermutoEncoding(torch.nn.Module):
     large tables and for inference.  float16 resolves the reference's initial values (about 1e-5)
     only to 6e-8; bfloat16 keeps three significant digits at any magnitude.
 
+    ``contiguous_output=True`` returns the (N, F(L+E)) result as a contiguous array instead of the strided
+    view the reference's permute + reshape produces (modules.py:87): for consumers that would otherwise
+    copy it (``torch.cat``, element-wise layers); a matrix multiplication takes the view as it is.
+
     ``sparse_table_grad=True`` is for tables that dwarf the batch: the gradient w.r.t. ``lattice_values``
     is not handed to autograd (``lattice_values.grad`` stays None) but added into ``table_grad``, a
     gradient array the module keeps across steps together with a map of the slot ranges that hold
@@ -33,9 +37,10 @@ class PermutoEncoding(torch.nn.Module):
 
     def __init__(self, pos_dim, capacity, nr_levels, nr_feat_per_level, scale_per_level,
                  appply_random_shift_per_level=True, concat_points=False, concat_points_scaling=1.0, device=None,
-                 lattice_half_precision=False, sparse_table_grad=False):
+                 lattice_half_precision=False, sparse_table_grad=False, contiguous_output=False):
         super().__init__()
         self.sparse_table_grad = bool(sparse_table_grad)
+        self.contiguous_output = bool(contiguous_output)
         if lattice_half_precision in (None, False):
             self.lattice_half_precision = None
         elif lattice_half_precision is True or lattice_half_precision == torch.float16:
@@ -84,6 +89,7 @@ class PermutoEncoding(torch.nn.Module):
         lattice = _native.EncodingWrapper.create(self.pos_dim, self.nr_feat_per_level, fixed_params)
         lattice.half_table = getattr(self, "lattice_half_precision", None)
         lattice.sparse_table_grad = getattr(self, "sparse_table_grad", False)
+        lattice.rows_output = getattr(self, "contiguous_output", False)
         return fixed_params, lattice
 
     @property

@@ -15,6 +15,12 @@ pays: output allocation, the loss, the gradient layout change and the optimiser 
 table.
 
     python -m permutohedral_encoding_amd.perf_sweep [--dims 2 3 4 5 6] [--points 524288] [--iters 300] [--fused-optimizer]
+
+``--consumers`` instead runs what the layer after the encoding does with the (N, 48) result of 2^20 points,
+a few times each and meant to be run under a kernel trace: ``torch.nn.Linear``, ``torch.cat`` with
+another (N, 3) array and an element-wise ``relu``, first on the module's default result (the strided
+view of the reference's permute + reshape, modules.py:87), then with ``contiguous_output=True``.  The
+trace shows which consumers copy the view and what the contiguous rows cost instead.
 """
 import argparse
 import json
@@ -69,6 +75,21 @@ def measure(pos_dim, nr_points, iters, warmup, levels=24, log2_capacity=18, fuse
     return res
 
 
+def consumers(nr_points=1 << 20, repeats=4):
+    lin = torch.nn.Linear(48, 32).cuda()
+    x = torch.rand(nr_points, 3, device="cuda")
+    other = torch.rand(nr_points, 3, device="cuda")
+    for contiguous in (False, True):
+        enc = PermutoEncoding(3, 1 << 18, 24, 2, np.geomspace(1.0, 1e-4, num=24), contiguous_output=contiguous)
+        with torch.no_grad():
+            for _ in range(repeats):
+                y = lin(enc(x))
+                z = torch.cat([enc(x), other], dim=1)
+                r = torch.relu(enc(x))
+        torch.cuda.synchronize()
+        print(f"contiguous_output={contiguous}: linear -> {tuple(y.shape)}, cat -> {tuple(z.shape)}, relu -> strides {r.stride()}")
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--dims", type=int, nargs="+", default=[2, 3, 4, 5, 6])
@@ -77,9 +98,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--fused-optimizer", action="store_true",
                     help="step the table with permutohedral_encoding_amd.optim.AdamW instead of torch.optim.AdamW")
+    ap.add_argument("--consumers", action="store_true", help="run the consumers of the forward result instead (for a kernel trace)")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("perf_sweep: no GPU visible; the encoding has no CPU path")
+    if args.consumers:
+        consumers()
+        return
     print("| pos_dim | inference (points/s) | training, table grad (points/s) | training, table + position grad (points/s) |")
     print("|---|---|---|---|")
     rows = []

@@ -561,3 +561,29 @@ def test_gradients_no_pass_consumes_are_not_computed():
     grad_pos, = torch.autograd.grad(sdf.sum(), pos, create_graph=True)
     ((grad_pos.norm(dim=1) - 1.0) ** 2).sum().backward()
     assert calls == [(False, True)] and doubles == [False]
+
+
+@pytest.mark.parametrize("d,feat,concat,n", [(3, 2, False, 5000), (4, 4, True, 777), (8, 2, True, 64), (2, 8, False, 10001)])
+def test_contiguous_output_equals_the_strided_view(d, feat, concat, n):
+    """penc_forward_rowmajor through PermutoEncoding(contiguous_output=True): the same bits as the default
+    (a strided view of the level-major result) in a contiguous (N, F(L+E)) array, gradients included."""
+    import permutohedral_encoding_amd as pe
+    levels = 6
+    sig = np.geomspace(1.0, 1e-2, levels)
+    torch.manual_seed(d)
+    plain = pe.PermutoEncoding(d, 1 << 12, levels, feat, sig, concat_points=concat, concat_points_scaling=0.5)
+    rows = pe.PermutoEncoding(d, 1 << 12, levels, feat, sig, concat_points=concat, concat_points_scaling=0.5, contiguous_output=True)
+    with torch.no_grad():
+        plain.lattice_values.uniform_(-1, 1)
+    rows.load_state_dict(plain.state_dict())
+    pos = torch.rand(n, d, device="cuda")
+    win = torch.tensor([1, 1, 0.5, 0, 1, 1], dtype=torch.float32)
+    pa, pb = pos.clone().requires_grad_(True), pos.clone().requires_grad_(True)
+    a, b = plain(pa, win), rows(pb, win)
+    assert b.is_contiguous() and not a.is_contiguous() and b.shape == a.shape == (n, plain.output_dims())
+    assert torch.equal(a, b)
+    up = torch.randn_like(b)
+    (a * up).sum().backward()
+    (b * up).sum().backward()
+    assert torch.allclose(pa.grad, pb.grad, rtol=1e-6, atol=1e-7 * pa.grad.abs().max().item())
+    assert torch.allclose(plain.lattice_values.grad, rows.lattice_values.grad, rtol=1e-5, atol=1e-6 * plain.lattice_values.grad.abs().max().item())
