@@ -283,12 +283,36 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
             }
         }
         const Located<D> s = locate<D>(pos, random_shift + level * D, scale_factor + level * D);
-        const uvec<D + 1> h = vertex_hashes<D>(s.rank, s.hash0);
+        uvec<D + 1> h;
         fvec<D + 1> w;  // b_r * w_level (:405), or dB[r] * w_level (:1244-1245)
-        if constexpr (kSecondOrder) {
-            w = pos_grad_grad_to_bary<D>(s.rank, q, scale_factor + level * D) * w_level;
+        bool via_lds = false;
+        if constexpr (D > kWorkgroupSortMaxDim) {
+            // Once the workgroup streams with every wave sorting on its own (stream_tile_wave), a wave's staging
+            // slice is idle between its tiles and nobody else touches it: it serves as the thread-private
+            // columns that put residuals and hash steps into rank order, in place of D(D+1) selects each
+            // (at D = 8 about 270 of 1350 vector instructions per point and level).
+            via_lds = mode == kModeStream && bins.n_bins <= static_cast<uint32_t>(kStageBins);
+        }
+        if (via_lds) {
+            constexpr uint32_t kSliceCells = ScatterStateT<stage_chunk(D)>::kChunk * 64 * 2;  // 8-byte cells of a wave's slice
+            static_assert((D + 1) * 64 <= kSliceCells, "a wave's staging slice holds a column of D+1 cells per lane");
+            uint2* const column = reinterpret_cast<uint2*>(state.val) + (threadIdx.x >> 6) * kSliceCells + (threadIdx.x & 63);
+            fvec<D + 1> sorted;
+            if constexpr (kSecondOrder) {
+                sort_by_rank_lds<D>(column, 64, s.rank, pos_grad_grad_to_elevated<D>(q, scale_factor + level * D), s.hash0, sorted, h);
+                w = sorted_elevated_grad_to_bary<D>(sorted) * w_level;
+            } else {
+                sort_by_rank_lds<D>(column, 64, s.rank, s.delta, s.hash0, sorted, h);
+                w = barycentric_of_sorted<D>(sorted) * w_level;
+            }
+            wave_lds_fence();  // the slice is staging space again from here on
         } else {
-            w = barycentric<D>(s.rank, s.delta) * w_level;
+            h = vertex_hashes<D>(s.rank, s.hash0);
+            if constexpr (kSecondOrder) {
+                w = pos_grad_grad_to_bary<D>(s.rank, q, scale_factor + level * D) * w_level;
+            } else {
+                w = barycentric<D>(s.rank, s.delta) * w_level;
+            }
         }
         uvec<D + 1> slot;
         static_for<D + 1>(PENC_BODY(r) {
