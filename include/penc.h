@@ -135,7 +135,7 @@ int penc_backward(int pos_dim, int nr_feat, int64_t nr_positions, int nr_levels,
  * PENC_STATIC_SCRATCH_BYTES inside the library's code object (one copy per GPU, held until the
  * process ends).  The call allocates and frees nothing.
  *   - Limit: one level's slot-range records must fit, i.e.
- *     penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels, capacity, 1) <= PENC_STATIC_SCRATCH_BYTES
+ *     penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels * nr_feat / 2, capacity, 1) <= PENC_STATIC_SCRATCH_BYTES
  *     (about 1.3 million points at pos_dim 3 and 2^18 slots, 0.7 million at 2^22 slots); larger problems return PENC_ERR_SCRATCH_TOO_SMALL
  *     and nothing is enqueued.  Levels are binned in as many passes as the scratch needs; position
  *     gradients whose partial sums do not fit are summed by one thread per point instead.

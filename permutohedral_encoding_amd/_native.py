@@ -337,6 +337,14 @@ class EncodingWrapper:
             self._half_copy_of = key
         return self._half_copy
 
+    def invalidate_half_table(self):
+        """Forgets the 16-bit copy, so that the next call converts the table again.  The copy follows the
+        tensor's version counter, which in-place operations under autograd's eyes and the bundled optimizers
+        advance; a write that bypasses it (``p.data.add_(...)``, a kernel given the raw pointer) does not,
+        and must be followed by this call."""
+        self._half_copy = None
+        self._half_copy_of = None
+
     def _check_common(self, inp):
         fp = self.fixed_params
         pos, lv, win = inp.m_positions_raw, inp.m_lattice_values, inp.m_anneal_window

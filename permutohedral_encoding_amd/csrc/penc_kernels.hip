@@ -1254,9 +1254,13 @@ int penc_backward_static(int pos_dim, int nr_feat, int64_t nr_positions, int nr_
                          void* stream) {
     if (int rc = check_geometry(pos_dim, nr_feat, nr_positions, nr_levels, capacity, 0)) return rc;
     // the scratch must hold the slot-range records of at least one level (more levels per pass as
-    // they fit); a capacity the scatter does not bin needs no scratch at all
-    if (lattice_values_grad != nullptr &&
-        penc_scatter_workspace_bytes(pos_dim, nr_positions, nr_levels, capacity, 1) > PENC_STATIC_SCRATCH_BYTES)
+    // they fit), a pair of features counting as a level; a problem the scatter does not bin (a capacity
+    // beyond the bins' reach, too few contributions per slot) needs no scratch at all
+    const int pair_levels = nr_levels * (nr_feat / 2);
+    const bool binned = bins_for_capacity(capacity) <= static_cast<uint32_t>(kMaxBins) &&
+                        nr_positions * (pos_dim + 1) * kMinSlotsPerContribution > capacity;
+    if (lattice_values_grad != nullptr && binned &&
+        penc_scatter_workspace_bytes(pos_dim, nr_positions, pair_levels, capacity, 1) > PENC_STATIC_SCRATCH_BYTES)
         return PENC_ERR_SCRATCH_TOO_SMALL;
     void* ws = static_scratch_of_current_device();
     if (ws == nullptr) return PENC_ERR_LAUNCH;

@@ -92,6 +92,22 @@ class PermutoEncoding(torch.nn.Module):
         lattice.rows_output = getattr(self, "contiguous_output", False)
         return fixed_params, lattice
 
+    def invalidate_half_table(self):
+        """With ``lattice_half_precision``: makes the next forward convert ``lattice_values`` again.  Needed only
+        after a write autograd's version counter does not see (``lattice_values.data.add_(...)``, a kernel
+        given the raw pointer); optimizer steps, ``load_state_dict``, ``.to()`` and ``train()``/``eval()``
+        are followed automatically."""
+        self.lattice.invalidate_half_table()
+
+    def train(self, mode=True):
+        self.lattice.invalidate_half_table()  # a cheap point at which a stale copy cannot survive
+        return super().train(mode)
+
+    def load_state_dict(self, *args, **kwargs):
+        out = super().load_state_dict(*args, **kwargs)
+        self.lattice.invalidate_half_table()
+        return out
+
     @property
     def table_grad(self):
         """With ``sparse_table_grad``: the ``SparseTableGrad`` the gradient calls add into (None before the first one)."""
@@ -110,6 +126,7 @@ class PermutoEncoding(torch.nn.Module):
     def _apply(self, fn, *args, **kwargs):
         # .to()/.cuda() replace the parameter tensors; the native handle must follow them
         out = super()._apply(fn, *args, **kwargs)
+        self.lattice.invalidate_half_table()
         self.anneal_window = fn(self.anneal_window)
         self.fixed_params.m_random_shift_per_level = self.random_shift_per_level
         return out

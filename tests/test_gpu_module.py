@@ -334,7 +334,7 @@ def test_row_major_backward_needs_room_for_the_copy():
     rc = lib.penc_backward_rowmajor(d, 2, n, levels, cap, t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(),
                                     t.data_ptr(), 8, t.data_ptr(), t.data_ptr(), ws.data_ptr(), 4096,
                                     torch.cuda.current_stream().cuda_stream)
-    assert rc == 8 and b"level-major copy" in lib.penc_status_string(rc)
+    assert rc == 8 and b"level-major array" in lib.penc_status_string(rc)
 
 
 @pytest.mark.parametrize("feat", [4, 8])
@@ -406,6 +406,12 @@ def test_module_gathers_from_a_half_precision_copy(switch, dtype):
     import pickle
     m2 = pickle.loads(pickle.dumps(m))
     assert m2.lattice_half_precision == dtype and torch.equal(m2(pos.detach()), out2)
+    # a write the version counter does not see leaves the copy stale until it is invalidated
+    m.lattice_values.data.mul_(2.0)
+    assert torch.equal(m(pos.detach()), out2)
+    m.invalidate_half_table()
+    want3 = orc.forward(p, narrow(t), sf, sh, w).transpose(2, 0, 1).reshape(n, -1)
+    assert np.array_equal(m(pos.detach()).detach().cpu().numpy(), want3)
 
 
 @pytest.mark.parametrize("n", [4096, 4099, 3])

@@ -19,18 +19,18 @@ orc = pytest.importorskip("oracle.api")
 SUM_RTOL = 1e-4
 
 
-def _both_entry_points(d, n, levels, cap, seed):
+def _both_entry_points(d, n, levels, cap, seed, feat=2):
     from permutohedral_encoding_amd import _native
     lib = _native.lib()
-    p = random_problem(d, n, levels, cap, seed=seed, sigma_range=(1.0, 1e-3))
+    p = random_problem(d, n, levels, cap, seed=seed, sigma_range=(1.0, 1e-3), nr_feat=feat)
     sf = orc.scale_factors(d, p["sigmas"])
-    enc, fp = make_encoding(d, p["sigmas"], p["shift"])
+    enc, fp = make_encoding(d, p["sigmas"], p["shift"], nr_feat=feat)
     pos, table, win, grad = to_gpu(p["pos"]), to_gpu(p["table"]), to_gpu(p["window"]), to_gpu(p["grad"])
     st = torch.cuda.current_stream().cuda_stream
-    common = (d, 2, n, levels, cap, pos.data_ptr(), table.data_ptr(), fp.m_scale_factor.data_ptr(),
+    common = (d, feat, n, levels, cap, pos.data_ptr(), table.data_ptr(), fp.m_scale_factor.data_ptr(),
               fp.m_random_shift_per_level.data_ptr(), win.data_ptr(), grad.data_ptr())
 
-    ws_bytes = max(int(lib.penc_scatter_workspace_bytes(d, n, levels, cap, 0)),
+    ws_bytes = max(int(lib.penc_scatter_workspace_bytes(d, n, levels * feat // 2, cap, 0)),
                    int(lib.penc_positions_workspace_bytes(d, n, levels)))
     ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device="cuda")
     tg_ref = torch.full_like(table, float("nan"))
@@ -39,11 +39,18 @@ def _both_entry_points(d, n, levels, cap, seed):
 
     tg = torch.full_like(table, float("nan"))
     pg = torch.full_like(pos, float("nan"))
+    # The entry point allocates nothing: neither through torch's caching allocator nor from the device
+    # directly.  The first call on a GPU looks up the scratch's address; the calls compared are later ones.
+    assert lib.penc_backward_static(*common, tg.data_ptr(), pg.data_ptr(), st) == 0
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    tg.fill_(float("nan"))
+    pg.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     assert lib.penc_backward_static(*common, tg.data_ptr(), pg.data_ptr(), st) == 0
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "the device's free memory changed across penc_backward_static"
 
     want = orc.backward_table(p["pos"], sf, p["shift"], p["window"], p["grad"], cap, want_abs=True)
     assert_sum_close(tg.cpu().numpy(), want["grad64"], want["abs64"], SUM_RTOL, "static-scratch table gradient vs oracle")
@@ -65,6 +72,8 @@ def test_static_scratch_backward_matches_the_workspace_entry_point_twice():
     assert torch.equal(pg, pg_ref)  # the partial sums fit the scratch here: same kernels, same order
     # and once more with another dimension and a capacity that is not a power of two
     _both_entry_points(5, 9_000, 5, 50_000, seed=103)
+    # four features per level: every pair of features is scattered like a level of its own
+    _both_entry_points(3, 120_000, 4, 1 << 16, seed=104, feat=4)
 
 
 def test_static_scratch_rejects_what_does_not_fit_and_enqueues_nothing():
