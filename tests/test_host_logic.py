@@ -69,6 +69,28 @@ def test_argument_validation_without_a_gpu():
     assert lib.penc_backward(3, 2, 10, 2, 16, p, z, p, p, p, p, z, p, None, 0, None) == 1
     assert lib.penc_double_backward_from_positions(3, 2, 10, 2, 16, p, p, p, p, p, p, p, z, z, 0, None, 0, None) == 1
     assert lib.penc_simplex_debug(3, 0, 2, 16, p, p, p, 0, z, z, z, z, None) == 2
+    # the sparse table gradient: gradient and map are both required; the map's size follows the slot ranges
+    assert lib.penc_backward_sparse(3, 2, 10, 2, 16, p, p, p, p, p, p, 0, p, z, z, None, 0, None) == 1
+    assert lib.penc_backward_sparse(3, 2, 10, 2, 16, p, p, p, p, p, p, 0, z, p, z, None, 0, None) == 1
+    assert lib.penc_backward_sparse(9, 2, 10, 2, 16, p, p, p, p, p, p, 0, p, p, z, None, 0, None) == 3
+    assert lib.penc_double_backward_from_positions_sparse(3, 2, 10, 2, 16, p, p, p, p, p, p, p, 0, p, z, p, 0, None, 0, None) == 1
+    assert lib.penc_double_backward_from_positions_sparse(3, 2, 10, 2, 16, p, p, p, p, p, p, p, 3, p, p, p, 0, None, 0, None) == 2  # odd row stride
+    assert lib.penc_touched_map_entries(2, 24, 1 << 18) == 24 * 32 and lib.penc_touched_range_slots(1 << 18) == 8192
+    assert lib.penc_touched_map_entries(8, 3, 1 << 22) == 3 * 4 * 512 and lib.penc_touched_range_slots(1 << 22) == 8192
+    assert lib.penc_touched_map_entries(2, 1, 1 << 24) == 512 and lib.penc_touched_range_slots(1 << 24) == 1 << 15
+    assert lib.penc_touched_map_entries(2, 5, 100003) == 5 * 13 and lib.penc_touched_map_entries(3, 5, 100) == 0
+    assert lib.penc_adamw_step_sparse(p, p, p, p, 2, 2, 16, z, 1e-3, 0.9, 0.99, 1e-8, 0.0, 1, 1, None) == 1
+    assert lib.penc_adamw_step_sparse(p, p, p, p, 2, 2, 16, p, 1e-3, 0.9, 0.99, 1e-8, 0.0, 0, 1, None) == 2  # steps count from 1
+    assert lib.penc_adamw_step_sparse(p, p, p, p, 3, 2, 16, p, 1e-3, 0.9, 0.99, 1e-8, 0.0, 1, 1, None) == 4
+    assert lib.penc_adamw_step_sparse(p, p + 4, p, p, 2, 2, 16, p, 1e-3, 0.9, 0.99, 1e-8, 0.0, 1, 1, None) == 5
+    assert lib.penc_clear_touched(z, 2, 2, 16, p, None) == 1 and lib.penc_clear_touched(p, 2, 0, 16, p, None) == 2
+    # dense rows from the forward: the workspace must hold the level-major array
+    assert lib.penc_forward_rowmajor(3, 2, 10, 2, 16, p, p, p, p, p, z, 4, 0, 1.0, p, 1 << 20, None) == 1
+    assert lib.penc_forward_rowmajor(3, 2, 10, 2, 16, p, p, p, p, p, p, 3, 0, 1.0, p, 1 << 20, None) == 2  # rows shorter than F * L
+    assert lib.penc_forward_rowmajor(3, 2, 10, 2, 16, p, p, p, p, p, p, 4, 0, 1.0, p, 16, None) == 8
+    assert lib.penc_forward_rowmajor(3, 2, 10, 2, 16, p, p, p, p, p, p, 4, 0, 1.0, None, 0, None) == 8
+    assert lib.penc_forward_rowmajor_workspace_bytes(3, 2, 10, 2, 0) == 4 * 2 * 2 * 10 + 256
+    assert lib.penc_forward_rowmajor_workspace_bytes(3, 2, 10, 2, 1) == 4 * 2 * 4 * 10 + 256
     # a table in half precision: slots of 2F bytes (4 for two features, 16 for eight)
     assert lib.penc_forward_half(3, 2, 10, 2, 16, p, p + 2, 1, p, p, p, p, 0, 1.0, None) == 5
     assert lib.penc_forward_half(3, 8, 10, 2, 16, p, p + 8, 2, p, p, p, p, 0, 1.0, None) == 5
