@@ -219,6 +219,9 @@ def run_probes(torch, capacity, n_threads, per_thread):
     dst = torch.empty_like(src)
     t = _timed(torch, lambda: lib.penc_probe_copy(src.data_ptr(), dst.data_ptr(), n4, st()))
     res["copy_GBps"] = 2 * n4 * 16 / t / 1e9
+    sink = torch.zeros(16384, dtype=torch.float32, device=dev)
+    t = _timed(torch, lambda: lib.penc_probe_read(src.data_ptr(), n4, sink.data_ptr(), st()))
+    res["read_GBps"] = n4 * 16 / t / 1e9
     del src, dst
 
     g = torch.Generator(device=dev)
@@ -563,7 +566,10 @@ def main():
             result["hbm_traffic_rate"] = {
                 "GBps": {k: per_phase[k] / (phase_ms[k] * 1e-3) / 1e9 for k in phase_ms if k in per_phase},
                 "copy_probe_GBps": pr["copy_GBps"],
-                "note": "HBM bytes per launch from hardware counters (profiles/) / measured phase time",
+                "read_probe_GBps": pr["read_GBps"],
+                "note": "bytes through the L2's memory-side port per launch from hardware counters (profiles/) / measured phase "
+                        "time; a phase that mostly reads is bounded by the read probe, one that reads and writes alike by the "
+                        "copy probe; part of the traffic of a table larger than the L2 is served by the memory-side cache",
             }
     if sparse and args.optimizer:
         def run_gradients():

@@ -7,6 +7,8 @@
  * (device pointers, a hipStream_t as void*, PENC_OK or a PENC_ERR_* code).
  *   copy   : dst[i] = src[i] for n_float4 16-byte elements (streaming bandwidth, and the known-size
  *            kernel that hardware byte counters are scaled by)
+ *   read   : reads n_float4 16-byte elements and writes at most one float per workgroup (`out` needs 16384 floats):
+ *            the streaming rate of a kernel that only reads, which a copy (half reads, half writes) does not reach
  *   gather : every thread sums `per_thread` (1..9) independent 8-byte loads table[idx[k][thread]] and
  *            writes one 8-byte result; idx holds per_thread * n_threads slots.  Fed with the slots a
  *            workload really uses (penc_simplex_debug), level by level, it measures what the gathers of
@@ -29,6 +31,7 @@ extern "C" {
 #endif
 
 int penc_probe_copy(const float* src, float* dst, int64_t n_float4, void* stream);
+int penc_probe_read(const float* src, int64_t n_float4, float* out, void* stream);
 int penc_probe_gather(const float* table, const int* idx, int64_t n_threads, int per_thread,
                       float* out, void* stream);
 int penc_probe_gather_variant(const float* table, int64_t table_slots, const int* idx, int64_t n_threads,

@@ -16,6 +16,17 @@ __global__ void __launch_bounds__(kBlock) copy_kernel(const float4* __restrict__
     for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
 }
 
+// Reads n4 16-byte elements and writes one value per workgroup: the streaming rate of a kernel that only reads.
+__global__ void __launch_bounds__(kBlock) read_kernel(const float4* __restrict__ src, size_t n4, float* __restrict__ out) {
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlock;
+    float acc = 0.0f;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlock + threadIdx.x; i < n4; i += stride) {
+        const float4 v = src[i];
+        acc += (v.x + v.y) + (v.z + v.w);
+    }
+    if (acc == 12345.678f) out[blockIdx.x] = acc;  // keeps the loads alive; practically never taken
+}
+
 // `per_thread` independent 8-byte loads per thread, indices coalesced across the wave
 // (idx[k][thread]), one 8-byte store: the access pattern of the forward pass without its arithmetic.
 template <int K>
@@ -123,6 +134,16 @@ int penc_probe_copy(const float* src, float* dst, int64_t n_float4, void* stream
     const unsigned blocks = static_cast<unsigned>(want < 16384 ? want : 16384);
     hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
                        reinterpret_cast<const float4*>(src), reinterpret_cast<float4*>(dst), static_cast<size_t>(n_float4));
+    return check_launch();
+}
+
+int penc_probe_read(const float* src, int64_t n_float4, float* out, void* stream) {
+    if (!src || !out) return PENC_ERR_NULL_POINTER;
+    if (n_float4 <= 0) return PENC_ERR_BAD_SIZE;
+    const int64_t want = (n_float4 + kBlock * 4 - 1) / (kBlock * 4);
+    const unsigned blocks = static_cast<unsigned>(want < 16384 ? want : 16384);
+    hipLaunchKernelGGL(read_kernel, dim3(blocks), dim3(kBlock), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<const float4*>(src), static_cast<size_t>(n_float4), out);
     return check_launch();
 }
 

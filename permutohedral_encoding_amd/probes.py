@@ -10,6 +10,7 @@ _lib = None
 _p = ctypes.c_void_p
 _SIGNATURES = {
     "penc_probe_copy": (ctypes.c_int, [_p, _p, ctypes.c_int64, _p]),
+    "penc_probe_read": (ctypes.c_int, [_p, ctypes.c_int64, _p, _p]),
     "penc_probe_gather": (ctypes.c_int, [_p, _p, ctypes.c_int64, ctypes.c_int, _p, _p]),
     "penc_probe_gather_variant": (ctypes.c_int, [_p, ctypes.c_int64, _p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                 ctypes.c_int, _p, _p]),

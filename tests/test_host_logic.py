@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
     handle = ctypes.CDLL(probes.LIB_PATH)
     for n in probe_names:
         assert hasattr(handle, n), f"{n} is declared in include/penc_probes.h but not exported"
-    assert set(probe_names) == set(probes.EXPORTED_SYMBOLS) and len(probe_names) == 4
+    assert set(probe_names) == set(probes.EXPORTED_SYMBOLS) and len(probe_names) == 5
 
 
 def test_status_strings_and_extra_levels():
