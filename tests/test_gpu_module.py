@@ -182,6 +182,63 @@ def test_forward_and_backward_replay_in_a_hip_graph():
         assert torch.allclose(tg_g, tg_eager, rtol=1e-4, atol=1e-6 * tg_eager.abs().max().item()), replay
 
 
+def test_sparse_training_step_replays_in_a_hip_graph():
+    """A whole sparse step (gradient call that adds and marks, optimizer step that updates, zeroes and
+    unmarks) is kernels on the given stream and nothing else: captured once and replayed, every replay
+    moves the table exactly like the same step run eagerly."""
+    from permutohedral_encoding_amd import _native
+    from helpers import random_problem, make_encoding
+    lib = _native.lib()
+    d, cap, levels, n = 3, 1 << 16, 6, 40000
+    p = random_problem(d, n, levels, cap, seed=33, sigma_range=(1.0, 2e-3))
+    enc, fp = make_encoding(d, p["sigmas"], p["shift"])
+    pos, win, grad = to_gpu(p["pos"]), to_gpu(p["window"]), to_gpu(p["grad"])
+    entries = int(lib.penc_touched_map_entries(2, levels, cap))
+    ws_bytes = int(lib.penc_scatter_workspace_bytes(d, n, levels, cap, 0))
+
+    def fresh():
+        return dict(table=to_gpu(p["table"]), m=torch.zeros(levels, cap, 2, device="cuda"), v=torch.zeros(levels, cap, 2, device="cuda"),
+                    g=torch.zeros(levels, cap, 2, device="cuda"), touched=torch.zeros(entries, dtype=torch.int32, device="cuda"),
+                    ws=torch.empty(ws_bytes, dtype=torch.uint8, device="cuda"))
+
+    def step(s, k):
+        st = torch.cuda.current_stream().cuda_stream
+        assert lib.penc_backward_sparse(d, 2, n, levels, cap, pos.data_ptr(), s["table"].data_ptr(), fp.m_scale_factor.data_ptr(),
+                                        fp.m_random_shift_per_level.data_ptr(), win.data_ptr(), grad.data_ptr(), 0, s["g"].data_ptr(),
+                                        s["touched"].data_ptr(), None, s["ws"].data_ptr(), ws_bytes, st) == 0
+        assert lib.penc_adamw_step_sparse(s["table"].data_ptr(), s["g"].data_ptr(), s["m"].data_ptr(), s["v"].data_ptr(), 2, levels, cap,
+                                          s["touched"].data_ptr(), 1e-2, 0.9, 0.99, 1e-8, 0.01, k, 1, st) == 0
+
+    eager = fresh()
+    snapshots = []
+    for k in range(3):  # the captured step keeps its step count: compare with eager steps that all use step 1
+        step(eager, 1)
+        torch.cuda.synchronize()
+        snapshots.append(eager["table"].clone())
+        assert not eager["g"].any().item() and not eager["touched"].any().item()
+
+    captured = fresh()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        warm = fresh()
+        step(warm, 1)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(captured, 1)
+    for k in range(3):
+        (grad * 2).sum().item()  # unrelated eager work and a synchronisation between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        scale = snapshots[k].abs().max().item()
+        assert torch.allclose(captured["table"], snapshots[k], rtol=1e-5, atol=1e-6 * scale), k
+        assert not captured["g"].any().item() and not captured["touched"].any().item()
+    assert free_before - torch.cuda.mem_get_info()[0] < (8 << 20)  # the capture itself allocated next to nothing
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 2), (255, 48), (256, 48), (257, 48), (100000, 32), (5000, 63), (7, 1), (1000, 255)])
 def test_streaming_transpose(rows, cols):
     from permutohedral_encoding_amd import _native
