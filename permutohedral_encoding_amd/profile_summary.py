@@ -90,6 +90,8 @@ def phase_of_dispatches(kernels):
             own.append("backward")
         elif b == "grad_grad_kernel":
             own.append("double_backward")
+        elif b == "touched_ranges_kernel":
+            own.append("clear_touched")
         elif b == "backward_table_kernel":
             args = template_args(k)  # <D, kRowMajor, kSecondOrder, kWideBins>
             own.append("double_backward" if len(args) >= 3 and args[2] == "true" else "backward")
@@ -149,18 +151,23 @@ def read_trace(base):
 
 
 def summarise(wl, digest, commit):
+    """`wl` is a workload of bench.py, or `<workload>_sparse` for its run with --sparse-table-grad (kernel trace only)."""
     base = os.path.join(ROOT, "gpurun_out", f"prof_{wl}")
     trace, bench = read_trace(base)
+    wl_name, _, variant = wl.partition("_")
+    flag = " --sparse-table-grad" if variant == "sparse" else ""
     with open(os.path.join(PROFILES, f"{wl}_kernel_trace.md"), "w") as f:
-        f.write(f"# Kernel trace: bench.py, workload {wl} ({DESCRIPTION[wl]}), one MI355X\n\n")
+        f.write(f"# Kernel trace: bench.py, workload {wl_name}{' with the sparse table gradient' if flag else ''} ({DESCRIPTION[wl_name]}), one MI355X\n\n")
         f.write("Command (from the repository root on the GPU box, after `cd /tmp && export TMPDIR=/tmp && cd -`):\n\n")
-        f.write(f"    rocprofv3 --kernel-trace --stats -f csv -d gpurun_out/prof_{wl}/trace -o run -- python3 bench.py --workload {wl} --no-cpu --no-probes --no-module --steps 20 --warmup 5\n\n")
+        f.write(f"    rocprofv3 --kernel-trace --stats -f csv -d gpurun_out/prof_{wl}/trace -o run -- python3 bench.py --workload {wl_name}{flag} --no-cpu --no-probes --no-module --steps 20 --warmup 5\n\n")
         f.write(f"Per phase of bench.py and kernel, over the run's dispatches (5 warm-up + 20 timed steps); kernel sources {digest} (commit {commit}):\n\n")
         f.write("| phase | kernel | calls | average (us) | min (us) | max (us) |\n|---|---|---|---|---|---|\n")
         for (ph, k), (avg, lo, hi, n) in sorted(trace.items(), key=lambda kv: (kv[0][0], -kv[1][0])):
             f.write(f"| {ph} | `{k}` | {n} | {avg:.1f} | {lo:.1f} | {hi:.1f} |\n")
         f.write(f"\nbench.py's own event timing in the same run: phases_ms = {json.dumps({k: round(v, 4) for k, v in bench['phases_ms'].items()})}, ms_per_step = {bench['ms_per_step']:.4f}.\n")
 
+    if variant:
+        return None  # a variant run has a kernel trace only
     sets = {name: read_counters(base, name) for name, _, _ in COUNTER_SETS}
     fetch, write, tcc, tcp, sq, ea = (sets[n] for n in ("fetch", "write", "tcc", "tcp", "sq", "ea"))
     known_kib = (1 << 30) / 1024.0  # the copy probe moves 1 GiB each way
@@ -239,7 +246,9 @@ def main(workloads):
                    "back in the same run) and wave-level vector instructions per launch (SQ_INSTS_VALU), per bench.py phase; every phase "
                    "lists the kernels it was summed over, and the rows of profiles/<workload>_counters.md hold the same figures")
     for wl in workloads:
-        cur[wl] = summarise(wl, digest, commit)
+        entry = summarise(wl, digest, commit)
+        if entry is not None:
+            cur[wl] = entry
     json.dump(cur, open(path, "w"), indent=1)
     print(json.dumps(cur, indent=1))
 
