@@ -319,7 +319,22 @@ backward_table_kernel(int n_points, int first_level, uint32_t n_pass_levels, uin
             PENC_INDEX(r);
             slot[r] = to_slot(h[r], capacity, cap_mask);
         });
-        if (t == 0) mode = scatter_mode_decide<D>(state, bins, active, slot, id_bits);
+        if (t == 0) {
+            // the next tile's slots, should the decision want to know whether its points use the slots this tile uses
+            // (its point is already here)
+            const auto slots_of_next_tile = [&]() {
+                const Located<D> s1 = locate<D>(pos_next, random_shift + level * D, scale_factor + level * D);
+                const uvec<D + 1> h1 = vertex_hashes<D>(s1.rank, s1.hash0);
+                uvec<D + 1> slot1;
+                static_for<D + 1>(PENC_BODY(r) {
+                    PENC_INDEX(r);
+                    slot1[r] = to_slot(h1[r], capacity, cap_mask);
+                });
+                return slot1;
+            };
+            const bool next_active = tile_base + kScatterBlock + threadIdx.x < n_points && tiles_per_group > 1;
+            mode = scatter_mode_decide<D>(state, bins, active, slot, id_bits, next_active, slots_of_next_tile, tiles_per_group);
+        }
         const uint32_t hits = scatter_tile<D>(state, level_grad, bins, group, active, cache_pays<D>(state, t),
                                               mode, id_bits, slot, w * g0, w * g1);  // g_f * (b_r * w_level), :405-410
         // the first tile finds the lines its own look-up has claimed: no evidence of reuse

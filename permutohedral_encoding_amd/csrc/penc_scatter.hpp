@@ -278,6 +278,48 @@ __device__ __forceinline__ void global_add_pairs(const GradSlice& level_grad, bo
     }
 }
 
+// Folds runs of neighbouring lanes that add to the same slot, within each row of 16 lanes: a segmented
+// inclusive scan over the row (DPP row shifts, four steps), after which the last lane of every run
+// holds the run's sums and is the only one of it still `live`.  Batches whose consecutive points are
+// neighbours in space (samples along a ray) make such runs at every level whose cells are wider than the
+// sampling distance: left alone they are what LDS atomics are slowest at (a few lanes on each of many
+// addresses, too few per address for the wave-wide fold below).  Returns the number of lanes folded away.
+// Must be called with all 64 lanes of the wave active.  Worth its 45 instructions only where many lanes have such a
+// neighbour: neighbours_share_slots() asks that of one vertex per tile, for all the tile's vertices.
+__device__ __forceinline__ bool neighbours_share_slots(uint32_t slot, bool live) {
+    const int key = live ? static_cast<int>(slot) : -1 - static_cast<int>(threadIdx.x & 63);
+    const int prev = __builtin_amdgcn_update_dpp(0, key, 0x111 /* row_shr:1 */, 0xf, 0xf, true);
+    return __popcll(__ballot((threadIdx.x & 15) != 0 && prev == key)) >= 16;
+}
+__device__ __forceinline__ uint32_t fold_adjacent_runs(uint32_t slot, bool& live, float& x0, float& x1) {
+    constexpr int kShr1 = 0x111, kShl1 = 0x101;  // row_shr:1, row_shl:1; row_shr:n is 0x110 + n
+    const uint32_t lane = threadIdx.x & 63, in_row = lane & 15;
+    // a lane that adds nothing gets a key of its own, so it joins no run
+    const int key = live ? static_cast<int>(slot) : -1 - static_cast<int>(lane);
+    const int prev = __builtin_amdgcn_update_dpp(0, key, kShr1, 0xf, 0xf, true);
+    // `open`: the partial sum of this lane does not reach back to the first lane of its run yet
+    int open = (in_row != 0 && prev == key) ? 1 : 0;
+#define PENC_SCAN_STEP(SHIFT)                                                                                              \
+    {                                                                                                                      \
+        const float s0 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x0), 0x110 + SHIFT, 0xf, 0xf, true)); \
+        const float s1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x1), 0x110 + SHIFT, 0xf, 0xf, true)); \
+        const int so = __builtin_amdgcn_update_dpp(0, open, 0x110 + SHIFT, 0xf, 0xf, true);  /* 0 from beyond the row: a run ends there */      \
+        x0 += open ? s0 : 0.0f;                                                                                            \
+        x1 += open ? s1 : 0.0f;                                                                                            \
+        open = open ? so : 0;                                                                                              \
+    }
+    PENC_SCAN_STEP(1)
+    PENC_SCAN_STEP(2)
+    PENC_SCAN_STEP(4)
+    PENC_SCAN_STEP(8)
+#undef PENC_SCAN_STEP
+    const int next = __builtin_amdgcn_update_dpp(0, key, kShl1, 0xf, 0xf, true);
+    const bool last_of_run = in_row == 15 || next != key;
+    const bool was_live = live;
+    live = live && last_of_run;
+    return __popcll(__ballot(was_live && !live));
+}
+
 // LDS state of a scattering workgroup.  The accumulate cache sums in fp64 with ds_add_f64: its
 // lines are hit by many lanes at once (that is what the cache is for), where a compare-and-swap
 // loop degrades quadratically (measured: 10-40x slower on the coarsest levels) and ds_add_f32 is
@@ -297,6 +339,7 @@ struct ScatterStateT {
     uint32_t wanted;               // contributions of the first tile
     uint32_t lines;                // lines they claimed: the tile's distinct slots, as far as the cache could take them
     uint32_t misses;               // contributions whose slot found no line
+    uint32_t strangers;            // slots of the second tile that the first tile did not touch (counted for levels with few slots)
 };
 
 template <typename State>
@@ -312,6 +355,7 @@ __device__ __forceinline__ void scatter_begin(State& c) {
         c.wanted = 0u;
         c.lines = 0u;
         c.misses = 0u;
+        c.strangers = 0u;
     }
     __syncthreads();
 }
@@ -356,6 +400,20 @@ __device__ __forceinline__ int cache_find(State& c, uint32_t slot, bool& found) 
         if (probe + 1 < kProbes) e = static_cast<int>((slot * kMix[probe]) >> (32 - kCacheLinesLog2));
     }
     return -1;
+}
+
+// Whether `slot` holds a line of the cache, without claiming one.
+template <int kProbes = 2, typename State>
+__device__ __forceinline__ bool cache_holds(const State& c, uint32_t slot) {
+    const int want = static_cast<int>(slot);
+    int e = static_cast<int>(slot & (kCacheLines - 1));
+    constexpr uint32_t kMix[3] = {0x9E3779B1u, 0x85EBCA6Bu, 0xC2B2AE35u};
+#pragma unroll
+    for (int probe = 0; probe < kProbes; ++probe) {
+        if (c.tag[e] == want) return true;
+        if (probe + 1 < kProbes) e = static_cast<int>((slot * kMix[probe]) >> (32 - kCacheLinesLog2));
+    }
+    return false;
 }
 
 // Stage 2 for a whole tile once the workgroup streams (see scatter_mode_decide): the cache's LDS is
@@ -782,6 +840,8 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
         return 0u;
     }
     uint32_t hits = 0;
+    // (wave-uniform) the points of this tile follow each other in space: neighbouring lanes often add to the same slot
+    const bool ordered = use_cache && neighbours_share_slots(slot[0], active);
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
         float x0 = a0[r], x1 = a1[r];
@@ -792,7 +852,9 @@ __device__ __forceinline__ uint32_t scatter_tile(State& c, const GradSlice& leve
             // kWaveGroups times, take the slot of the first pending lane, sum the contributions of
             // all lanes that share it with DPP, and leave the sum with that lane alone.  A group
             // of fewer than kMinWaveGroup lanes means the wave's slots are spread out: stop.
-            unsigned long long pending = __ballot(active);
+            // neighbouring lanes on one slot first (points that follow each other in space), then the slots most of the wave shares
+            if (ordered) hits += fold_adjacent_runs(slot[r], miss, x0, x1);
+            unsigned long long pending = __ballot(miss);
 #pragma unroll 1
             for (int round = 0; round < kWaveGroups && pending != 0ull; ++round) {
                 const int leader = __builtin_ctzll(pending);
@@ -875,9 +937,10 @@ __device__ __forceinline__ void cache_flush(State& c, const GradSlice& level_gra
 // that would not hit is never filled: its LDS becomes staging space (kModeStream, see
 // stream_tile; needs bins).  One that hits on at most 64 lines becomes columns (kModeColumns,
 // `id_bits` says how many).  Otherwise the cache serves, with the lines already claimed.
-template <int D, typename State>
+template <int D, typename State, typename NextSlots>
 __device__ __forceinline__ int scatter_mode_decide(State& c, const BinTarget& bins, bool active, uvec<D + 1> slot,
-                                                   uint32_t& id_bits) {
+                                                   uint32_t& id_bits, bool next_active, NextSlots&& slots_of_next_tile,
+                                                   int tiles_per_group) {
     uint32_t wanted = 0, missed = 0;  // over the wave
     static_for<D + 1>(PENC_BODY(r) {
         PENC_INDEX(r);
@@ -894,16 +957,35 @@ __device__ __forceinline__ int scatter_mode_decide(State& c, const BinTarget& bi
     uint32_t used = 0;
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) used += __popcll(__ballot(c.tag[e] != -1));
     if ((threadIdx.x & 63) == 0 && used != 0u) atomicAdd(&c.lines, used);
+    // Columns are for a level whose few slots the whole group shares.  The first tile shows that when the points come in no
+    // particular order; where they follow each other in space (every tile another ray) each tile brings slots of its own, the
+    // table of columns fills up, and every contribution that then finds no column probes in vain and leaves one record.  The
+    // second tile's slots tell the two apart: how many of them did the first tile not touch?
+    // (asked only of a level that is a candidate for columns: the look at the second tile costs a simplex search)
     __syncthreads();
+    if (cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1)) &&
+        c.lines * static_cast<uint32_t>(tiles_per_group) > (1u << kColumnMaxIdsLog2)) {
+        const uvec<D + 1> next_slot = slots_of_next_tile();
+        uint32_t strangers = 0;
+        static_for<D + 1>(PENC_BODY(r) {
+            PENC_INDEX(r);
+            strangers += __popcll(__ballot(next_active && !cache_holds(c, next_slot[r])));
+        });
+        if ((threadIdx.x & 63) == 0 && strangers != 0u) atomicAdd(&c.strangers, strangers);
+        __syncthreads();
+    }
     int mode = kModeCache;
     const bool can_stream = bins.records != nullptr && bins.n_bins <= static_cast<uint32_t>(kMaxBins);
+    // with a fresh set of slots in every tile, columns only if as many slots again from every later tile would still fit
+    const bool fresh_slots_per_tile = c.strangers * 4u > c.wanted;
     if (can_stream && !cache_pays<D>(c, 0, 4u)) {
         mode = kModeStream;
         if (bins.n_bins > kStageBins) {  // stream_tile_many wants its per-bin counters cleared
             for (int e = threadIdx.x; e < kMaxBins; e += kScatterBlock) c.tag[e] = 0;
             __syncthreads();
         }
-    } else if (cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1))) {  // the table of columns starts at most half full
+    } else if (cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1)) &&  // the table of columns starts at most half full
+               (!fresh_slots_per_tile || c.lines * static_cast<uint32_t>(tiles_per_group) <= (1u << kColumnMaxIdsLog2))) {
         mode = kModeColumns;
         id_bits = kColumnMinIdsLog2;
         while ((1u << (id_bits - 1)) < c.lines) ++id_bits;

@@ -20,7 +20,7 @@ class Workload:
     nr_levels: int
     nr_points: int
     scale_range: Tuple[float, float]
-    points: str = "uniform"  # "uniform" in [0,1]^D or "sphere" (shell of radius 0.5 around 0.5)
+    points: str = "uniform"  # "uniform" in [0,1]^D, "sphere" (shell of radius 0.5 around 0.5) or "rays" (samples along chords, in order)
     masked_top_levels: int = 0  # anneal window = 1 for the coarse levels, 0 for this many fine ones
     phases: Tuple[str, ...] = field(default=("forward",))
 
@@ -41,7 +41,12 @@ WORKLOADS = {
     "c4": Workload("c4", 8, 1 << 19, 16, 1 << 19, (1.0, 1e-3), phases=("forward", "backward_table")),
     "c5": Workload("c5", 3, 1 << 22, 24, 1 << 20, (1.0, 1e-4), points="sphere", masked_top_levels=8,
                    phases=("forward", "backward_table", "backward_pos", "double_backward")),
+    # not a BASELINE configuration: c2 with the points a renderer hands over, 128 consecutive samples along each of
+    # 8192 rays, so that neighbouring points are neighbours in space (the benchmark's uniform points never are)
+    "c2_rays": Workload("c2_rays", 3, 1 << 18, 24, 1 << 20, (1.0, 1e-4), points="rays", phases=("forward", "backward_table")),
 }
+
+RAY_SAMPLES = 128
 
 
 def scale_list(w: Workload):
@@ -78,6 +83,15 @@ def make_inputs(w: Workload, need=("table", "shift", "pos", "grad", "dpos"), nr_
             u /= np.linalg.norm(u, axis=1, keepdims=True)
             r = 0.5 + rng.standard_normal((n, 1)) * 0.02
             out["pos"] = (0.5 + r * u).astype(np.float32)
+        elif w.points == "rays":
+            rng = np.random.default_rng(7)
+            n_rays = (n + RAY_SAMPLES - 1) // RAY_SAMPLES
+            origin = rng.uniform(0.25, 0.75, (n_rays, d))
+            direction = rng.standard_normal((n_rays, d))
+            direction /= np.linalg.norm(direction, axis=1, keepdims=True)
+            along = (np.arange(RAY_SAMPLES) + rng.uniform(0, 1, (n_rays, RAY_SAMPLES))) / RAY_SAMPLES - 0.5  # stratified
+            pos = origin[:, None, :] + 0.8 * along[:, :, None] * direction[:, None, :]
+            out["pos"] = np.clip(pos.reshape(-1, d)[:n], 0.0, 1.0).astype(np.float32)
         else:
             raise ValueError(w.points)
     if "grad" in need:

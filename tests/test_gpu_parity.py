@@ -728,6 +728,34 @@ def test_table_gradients_on_mixed_point_distributions(seed):
     _table_gradients_match(p, d, cap, f"seed {seed}: D={d} cap={cap} n={n} clusters={n_clusters}")
 
 
+@pytest.mark.parametrize("d,samples,n,cap", [(3, 512, 70000, 1 << 18), (3, 128, 50000, 1 << 16), (4, 64, 40000, 1 << 18),
+                                             (2, 1024, 60000, 1 << 14), (6, 256, 30000, 1 << 18), (3, 7, 30000, 30011)])
+def test_table_gradients_on_points_in_spatial_order(d, samples, n, cap):
+    """Batches whose consecutive points are neighbours in space: samples along rays (a tile of 512 points is one
+    ray, a few rays, or many short ones) and points sorted along a space-filling curve.  Neighbouring lanes then add
+    to the same slots (the fold of adjacent runs), every tile brings slots of its own (column mode must not be
+    chosen from the first tile alone), and the first and second order table gradients must still be the oracle's."""
+    levels = 7
+    rng = np.random.default_rng(500 + d + samples)
+    p = random_problem(d, n, levels, cap, seed=600 + d, sigma_range=(1.0, 3e-3))
+    n_rays = (n + samples - 1) // samples
+    origin = rng.uniform(0.2, 0.8, (n_rays, d))
+    direction = rng.standard_normal((n_rays, d))
+    direction /= np.linalg.norm(direction, axis=1, keepdims=True)
+    along = (np.arange(samples) + rng.uniform(0, 1, (n_rays, samples))) / samples - 0.5
+    rays = (origin[:, None, :] + 0.6 * along[:, :, None] * direction[:, None, :]).reshape(-1, d)[:n]
+    p["pos"] = rays.astype(np.float32)
+    _table_gradients_match(p, d, cap, f"rays of {samples} samples, D={d}")
+    # the same points along a Z-order curve: neighbours in space without being runs along a line
+    q = np.clip((rays * 256).astype(np.int64), 0, 255)
+    key = np.zeros(n, np.int64)
+    for bit in range(8):
+        for k in range(d):
+            key |= ((q[:, k] >> bit) & 1) << (bit * d + k)
+    p["pos"] = rays[np.argsort(key, kind="stable")].astype(np.float32)
+    _table_gradients_match(p, d, cap, f"Z-order, D={d}")
+
+
 def test_segments_overflow_with_more_bins_than_lanes():
     """The same deception on a 2^20-slot table (128 slot ranges: the tile is sorted with one counter and
     one thread per bin): the first 512 points of every group are spread out, all the others sit in one

@@ -206,6 +206,10 @@ def test_workloads_are_seeded_and_shaped():
     r = np.linalg.norm(s - 0.5, axis=1)
     assert abs(r.mean() - 0.5) < 5e-3 and 0.015 < r.std() < 0.025
     assert workloads.WORKLOADS["c2"].point_levels == 25165824
+    # the ray-ordered variant of c2: consecutive points are consecutive samples of one ray
+    rays = workloads.make_inputs(workloads.WORKLOADS["c2_rays"].scaled(1024), need=("pos",))["pos"]
+    step = np.linalg.norm(np.diff(rays.reshape(8, 128, 3), axis=1), axis=2)
+    assert rays.shape == (1024, 3) and rays.min() >= 0 and rays.max() <= 1 and step.max() < 0.02
 
 
 def test_workspace_request_is_capped_and_shrinks_when_memory_runs_out(monkeypatch):
