@@ -958,13 +958,14 @@ __device__ __forceinline__ int scatter_mode_decide(State& c, const BinTarget& bi
     for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) used += __popcll(__ballot(c.tag[e] != -1));
     if ((threadIdx.x & 63) == 0 && used != 0u) atomicAdd(&c.lines, used);
     // Columns are for a level whose few slots the whole group shares.  The first tile shows that when the points come in no
-    // particular order; where they follow each other in space (every tile another ray) each tile brings slots of its own, the
-    // table of columns fills up, and every contribution that then finds no column probes in vain and leaves one record.  The
-    // second tile's slots tell the two apart: how many of them did the first tile not touch?
-    // (asked only of a level that is a candidate for columns: the look at the second tile costs a simplex search)
+    // particular order; where they follow each other in space (every tile another ray, or the next stretch of a space-filling
+    // curve) each tile brings slots of its own, the table of columns fills up, and every contribution that then finds no
+    // column probes in vain and leaves one record.  The second tile's slots tell the two apart: how many of its contributions
+    // go to slots the first tile did not touch?  (Asked only of a level that is a candidate for columns: the look at the
+    // second tile costs a simplex search.)
     __syncthreads();
-    if (cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1)) &&
-        c.lines * static_cast<uint32_t>(tiles_per_group) > (1u << kColumnMaxIdsLog2)) {
+    const bool few_slots = cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1));  // the table of columns starts at most half full
+    if (few_slots && tiles_per_group > 1) {
         const uvec<D + 1> next_slot = slots_of_next_tile();
         uint32_t strangers = 0;
         static_for<D + 1>(PENC_BODY(r) {
@@ -976,19 +977,20 @@ __device__ __forceinline__ int scatter_mode_decide(State& c, const BinTarget& bi
     }
     int mode = kModeCache;
     const bool can_stream = bins.records != nullptr && bins.n_bins <= static_cast<uint32_t>(kMaxBins);
-    // with a fresh set of slots in every tile, columns only if as many slots again from every later tile would still fit
-    const bool fresh_slots_per_tile = c.strangers * 4u > c.wanted;
+    // The slots the group will have touched in the end: the first tile's, and from every later tile as many new ones as the
+    // second tile brought, counted twice (a slot at the rim of what a tile covers gets fewer contributions than one inside).
+    const uint32_t expected_slots =
+        c.lines + (2u * c.lines * c.strangers * static_cast<uint32_t>(tiles_per_group - 1)) / (c.wanted != 0u ? c.wanted : 1u);
     if (can_stream && !cache_pays<D>(c, 0, 4u)) {
         mode = kModeStream;
         if (bins.n_bins > kStageBins) {  // stream_tile_many wants its per-bin counters cleared
             for (int e = threadIdx.x; e < kMaxBins; e += kScatterBlock) c.tag[e] = 0;
             __syncthreads();
         }
-    } else if (cache_pays<D>(c, 0) && c.lines <= (1u << (kColumnMaxIdsLog2 - 1)) &&  // the table of columns starts at most half full
-               (!fresh_slots_per_tile || c.lines * static_cast<uint32_t>(tiles_per_group) <= (1u << kColumnMaxIdsLog2))) {
+    } else if (few_slots && expected_slots <= (3u << (kColumnMaxIdsLog2 - 2))) {  // the largest table may end up three quarters full
         mode = kModeColumns;
         id_bits = kColumnMinIdsLog2;
-        while ((1u << (id_bits - 1)) < c.lines) ++id_bits;
+        while ((1u << (id_bits - 1)) < expected_slots && id_bits < static_cast<uint32_t>(kColumnMaxIdsLog2)) ++id_bits;
         for (int e = threadIdx.x; e < kCacheLines; e += kScatterBlock) c.tag[e] = -1;  // now the table of columns
         __syncthreads();
     }
