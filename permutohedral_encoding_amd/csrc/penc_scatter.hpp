@@ -198,8 +198,10 @@ struct GradSlice {
     uint32_t* direct;
     uint32_t bin_shift;  // of the bins `direct` belongs to
     __device__ __forceinline__ float* at(uint32_t slot) const { return base + static_cast<size_t>(slot) * slot_floats; }
+    // Many workgroups may set the same flag at once, all to 1, and nobody reads it before the kernel ends: a relaxed
+    // atomic store (an ordinary store instruction) says so.
     __device__ __forceinline__ void mark_direct(uint32_t slot) const {
-        if (direct != nullptr) direct[slot >> bin_shift] = 1u;
+        if (direct != nullptr) __hip_atomic_store(&direct[slot >> bin_shift], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 };
 
@@ -935,8 +937,9 @@ __device__ __forceinline__ void cache_flush(State& c, const GradSlice& level_gra
 // whole workgroup how the level goes.  The slots are looked up in the (empty) cache, which claims a
 // line for every distinct slot as far as it can; the counts tell what the cache is good for.  One
 // that would not hit is never filled: its LDS becomes staging space (kModeStream, see
-// stream_tile; needs bins).  One that hits on at most 64 lines becomes columns (kModeColumns,
-// `id_bits` says how many).  Otherwise the cache serves, with the lines already claimed.
+// stream_tile; needs bins).  One that hits on at most 64 lines, and whose group of points is not expected to
+// touch more than 96 slots in all, becomes columns (kModeColumns, `id_bits` says how many).  Otherwise the
+// cache serves, with the lines already claimed.
 template <int D, typename State, typename NextSlots>
 __device__ __forceinline__ int scatter_mode_decide(State& c, const BinTarget& bins, bool active, uvec<D + 1> slot,
                                                    uint32_t& id_bits, bool next_active, NextSlots&& slots_of_next_tile,
