@@ -198,10 +198,11 @@ struct GradSlice {
     uint32_t* direct;
     uint32_t bin_shift;  // of the bins `direct` belongs to
     __device__ __forceinline__ float* at(uint32_t slot) const { return base + static_cast<size_t>(slot) * slot_floats; }
-    // Many workgroups may set the same flag at once, all to 1, and nobody reads it before the kernel ends: a relaxed
-    // atomic store (an ordinary store instruction) says so.
+    // A plain store on purpose: many workgroups may set the same flag at once, all to 1, and nobody reads it before the
+    // kernel has ended.  (As a relaxed atomic store of device scope, a store that writes through the L2, the levels that
+    // sum in columns took up to 2.5 times as long and the kernel 8% longer.)
     __device__ __forceinline__ void mark_direct(uint32_t slot) const {
-        if (direct != nullptr) __hip_atomic_store(&direct[slot >> bin_shift], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (direct != nullptr) direct[slot >> bin_shift] = 1u;
     }
 };
 
