@@ -485,6 +485,55 @@ def test_full_size_adjoint_identities(name):
     assert torch.allclose(tg2, tg2_direct, rtol=1e-3, atol=1e-5 * tg2.abs().max().item())
 
 
+@pytest.mark.parametrize("name", ["c2", "c3"])
+def test_full_size_table_gradients_do_not_depend_on_the_order_of_the_points(name):
+    """A permutation of the batch permutes nothing in the table gradient.  The scatter treats an ordered batch
+    differently at every level (folded runs of neighbouring lanes, columns sized from the second tile, the
+    accumulate cache where unordered points stream), so equal sums for the benchmark's unordered points, the same
+    points along a Z-order curve and the same points sorted by their first coordinate check those paths at the
+    full size.  Bound per slot: 1e-5 of the sum of the magnitudes of its terms (first order: that sum is the
+    gradient of |g|, since the barycentric weights are not negative), and 2e-5 of the level's largest entry
+    for the second order, whose weights have both signs."""
+    from permutohedral_encoding_amd import _native
+    w = wl.WORKLOADS[name]
+    p = wl.make_inputs(w)
+    enc, _ = make_encoding(w.pos_dim, p["sigmas"], p["shift"])
+    table_t = torch.zeros((w.nr_levels, w.capacity, 2), device="cuda")
+    win_t = to_gpu(p["window"])
+    second = "double_backward" in w.phases
+
+    def gradients(order, grad):
+        pos_t = to_gpu(np.ascontiguousarray(p["pos"][order]))
+        grad_t = to_gpu(np.ascontiguousarray(grad[:, :, order]))
+        inp = _native.EncodingInput(table_t, pos_t, win_t, True, False)
+        tg, _ = enc.backward(inp, grad_t)
+        tg2 = None
+        if second:
+            tg2, _ = enc.double_backward_from_positions(_native.EncodingInput(table_t, pos_t, win_t, True, True),
+                                                        to_gpu(np.ascontiguousarray(p["dpos"][order])), grad_t)
+        return tg.double(), None if tg2 is None else tg2.double()
+
+    n, d = w.nr_points, w.pos_dim
+    cells = np.clip((p["pos"] * 256).astype(np.int64), 0, 255)
+    key = np.zeros(n, np.int64)
+    for bit in range(8):
+        for k in range(d):
+            key |= ((cells[:, k] >> bit) & 1) << (bit * d + k)
+    orders = {"Z-order": np.argsort(key, kind="stable"), "sorted by x": np.argsort(p["pos"][:, 0], kind="stable"),
+              "reversed": np.arange(n)[::-1].copy()}
+    identity = np.arange(n)
+    base, base2 = gradients(identity, p["grad"])
+    magnitude, _ = gradients(identity, np.abs(p["grad"]))
+    for what, order in orders.items():
+        got, got2 = gradients(order, p["grad"])
+        excess = (torch.abs(got - base) - (1e-5 * magnitude + 1e-30)).max().item()
+        assert excess <= 0.0, f"{name}, {what}: first-order table gradient differs by {excess:.3g} beyond the bound"
+        if second:
+            level_scale = base2.abs().amax(dim=(1, 2), keepdim=True)
+            excess2 = (torch.abs(got2 - base2) - (2e-5 * level_scale + 1e-30)).max().item()
+            assert excess2 <= 0.0, f"{name}, {what}: second-order table gradient differs by {excess2:.3g} beyond the bound"
+
+
 def test_full_size_constant_table_gives_window():
     w = wl.WORKLOADS["c2"]
     p = wl.make_inputs(w, need=("shift", "pos"))
