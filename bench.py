@@ -276,14 +276,13 @@ def gather_pattern_seconds(torch, native, w, fp, table, pos, variant=None):
     out = torch.empty(n * 2, dtype=torch.float32, device="cuda")
     zeros = torch.zeros((d + 1, n), dtype=torch.int32, device="cuda")
     level_table = table[0]
-    t_zero = _timed(torch, lambda: plib.penc_probe_gather(level_table.data_ptr(), zeros.data_ptr(), n, d + 1, out.data_ptr(), st), iters=10)
-    t_zero_variant = None
+    run_default = lambda idx_: plib.penc_probe_gather(level_table.data_ptr(), idx_.data_ptr(), n, d + 1, out.data_ptr(), st)
+    run_variant = None
     if variant is not None:
         run_variant = lambda idx_: plib.penc_probe_gather_variant(level_table.data_ptr(), cap, idx_.data_ptr(), n, d + 1, variant[0],
                                                                   variant[1], variant[2], out.data_ptr(), st)
-        t_zero_variant = _timed(torch, lambda: run_variant(zeros), iters=10)
     slot = torch.empty((1, n, d + 1), dtype=torch.int32, device="cuda")
-    result = []
+    real, real_variant, zero, zero_variant = [], [], [], []
     for l in range(levels):
         rc = lib.penc_simplex_debug(d, n, 1, cap, pos.data_ptr(), fp.m_scale_factor[l:l + 1].contiguous().data_ptr(),
                                     fp.m_random_shift_per_level[l:l + 1].contiguous().data_ptr(), 1, None, None,
@@ -291,11 +290,18 @@ def gather_pattern_seconds(torch, native, w, fp, table, pos, variant=None):
         assert rc == 0, rc
         idx = slot[0].t().contiguous()
         level_table = table[l]
-        t_real = _timed(torch, lambda: plib.penc_probe_gather(level_table.data_ptr(), idx.data_ptr(), n, d + 1, out.data_ptr(), st), iters=10)
-        cost = max(t_real - t_zero, 0.0)
-        if variant is not None:
-            cost = min(cost, max(_timed(torch, lambda: run_variant(idx), iters=10) - t_zero_variant, 0.0))
-        result.append(cost)
+        real.append(_timed(torch, lambda: run_default(idx), iters=10))
+        # the all-hit run is repeated beside every level and its median is what is subtracted: taken once, its
+        # half-microsecond scatter would shift every level of the bound the same way
+        zero.append(_timed(torch, lambda: run_default(zeros), iters=10))
+        if run_variant is not None:
+            real_variant.append(_timed(torch, lambda: run_variant(idx), iters=10))
+            zero_variant.append(_timed(torch, lambda: run_variant(zeros), iters=10))
+    t_zero = float(np.median(zero))
+    result = [max(t - t_zero, 0.0) for t in real]
+    if run_variant is not None:
+        t_zero_variant = float(np.median(zero_variant))
+        result = [min(c, max(t - t_zero_variant, 0.0)) for c, t in zip(result, real_variant)]
     return result, t_zero
 
 
