@@ -14,7 +14,7 @@ Unlike the kernel benchmark (``bench.py``) these figures include everything a us
 pays: output allocation, the loss, the gradient layout change and the optimiser walking the whole
 table.
 
-    python -m permutohedral_encoding_amd.perf_sweep [--dims 2 3 4 5 6] [--points 524288] [--iters 300] [--fused-optimizer]
+    python -m permutohedral_encoding_amd.perf_sweep [--dims 2 3 4 5 6] [--points 524288] [--iters 300] [--fused-optimizer] [--contiguous-output]
 
 ``--consumers`` instead runs what the layer after the encoding does with the (N, 48) result of 2^20 points,
 a few times each and meant to be run under a kernel trace: ``torch.nn.Linear``, ``torch.cat`` with
@@ -51,9 +51,10 @@ def _timed(step, nr_points, iters, warmup):
     return float(np.mean(kept))
 
 
-def measure(pos_dim, nr_points, iters, warmup, levels=24, log2_capacity=18, fused_optimizer=False):
+def measure(pos_dim, nr_points, iters, warmup, levels=24, log2_capacity=18, fused_optimizer=False, contiguous_output=False):
     torch.manual_seed(0)
-    enc = PermutoEncoding(pos_dim, 1 << log2_capacity, levels, 2, np.geomspace(1.0, 1e-4, num=levels))
+    enc = PermutoEncoding(pos_dim, 1 << log2_capacity, levels, 2, np.geomspace(1.0, 1e-4, num=levels),
+                          contiguous_output=contiguous_output)
     if fused_optimizer:  # the library's one-kernel AdamW instead of torch's (same update)
         from .optim import AdamW
         opt = AdamW(enc.parameters(), betas=(0.9, 0.99), eps=1e-15, weight_decay=0.0, lr=1e-3)
@@ -183,6 +184,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--fused-optimizer", action="store_true",
                     help="step the table with permutohedral_encoding_amd.optim.AdamW instead of torch.optim.AdamW")
+    ap.add_argument("--contiguous-output", action="store_true",
+                    help="build the module with contiguous_output=True: dense (N, F*L) rows instead of the strided view")
     ap.add_argument("--consumers", action="store_true", help="run the consumers of the forward result instead (for a kernel trace)")
     ap.add_argument("--point-orders", action="store_true", help="time forward and table backward on unordered, ray-ordered and Z-ordered points instead")
     args = ap.parse_args()
@@ -198,7 +201,8 @@ def main():
     print("|---|---|---|---|")
     rows = []
     for d in args.dims:
-        r = measure(d, args.points, args.iters, args.warmup, fused_optimizer=args.fused_optimizer)
+        r = measure(d, args.points, args.iters, args.warmup, fused_optimizer=args.fused_optimizer,
+                    contiguous_output=args.contiguous_output)
         rows.append(r)
         print(f"| {d} | {r['inference']:.3g} | {r['train_table']:.3g} | {r['train_table_pos']:.3g} |", flush=True)
     print(json.dumps(rows))
