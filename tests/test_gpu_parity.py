@@ -969,13 +969,29 @@ def _random_geometry(seed):
 
 @pytest.mark.parametrize("seed", range(20))
 def test_random_geometry_all_phases_match_oracle(seed, monkeypatch):
-    """Twenty seeded random problems through every phase against the oracle.  Run under -x the suite
-    stops at the first geometry that disagrees; the assertion message names it."""
+    """Twenty seeded random problems through every phase against the oracle, the points unordered or in one of three
+    orders.  Run under -x the suite stops at the first geometry that disagrees; the assertion message names it."""
     from permutohedral_encoding_amd import _native
     g = _random_geometry(seed)
     d, feat, cap, n, levels = g["d"], g["feat"], g["cap"], g["n"], g["levels"]
     what = f"seed {seed}: {g}"
     p = random_problem(d, n, levels, 1, seed=g["problem_seed"], sigma_range=(1.0, g["sigma_lo"]), nr_feat=feat)
+    # three seeds in four hand the points over in an order: along a Z-order curve, sorted by their first coordinate,
+    # or in runs of identical points (the scatter folds neighbouring lanes and sizes its column tables from the second tile)
+    order = seed % 4
+    if order == 1:
+        cells = np.clip((p["pos"] * 256).astype(np.int64), 0, 255)
+        key = np.zeros(n, np.int64)
+        for bit in range(7):
+            for k in range(d):
+                key |= ((cells[:, k] >> bit) & 1) << (bit * d + k)
+        p["pos"] = np.ascontiguousarray(p["pos"][np.argsort(key, kind="stable")])
+    elif order == 2:
+        p["pos"] = np.ascontiguousarray(p["pos"][np.argsort(p["pos"][:, 0], kind="stable")])
+    elif order == 3:
+        run = int(np.random.default_rng(seed).choice([2, 7, 64, 700]))
+        p["pos"] = np.ascontiguousarray(np.repeat(p["pos"][: (n + run - 1) // run], run, axis=0)[:n])
+    what += f", point order {order}"
     if g["masked"] is not None:
         p["window"][g["masked"]] = 0.0
     p["table"] = np.random.default_rng(g["problem_seed"] + 1).uniform(-1, 1, (levels, cap, feat)).astype(np.float32)
